@@ -350,7 +350,7 @@ __global__ __launch_bounds__(NW * 64) void dgemv_mx_kernel(const DgArgs a) {
 // Which launches run here (GBX_DG_MX: 0 none, 1 the SwiGLU launches = gate|up, 2 every eligible launch)
 bool dg_mx_wanted(const DgArgs& a, const DgPlan& pl, int epi, bool bf16) {
   static const int mode = env_switch("GBX_DG_MX");
-  // (K = 8192 -- four spans of operands in registers -- builds with > 100 spilled registers at 16 waves per CU: scratch/kernel_resources.py;
+  // (K = 8192 -- four spans of operands in registers -- builds with > 100 spilled registers at 16 waves per CU;
   //  those launches stay on the vector form)
   if (!mode || !bf16 || pl.KS != 1 || pl.R != 2 || a.log2g != 7 || (a.K % 2048) != 0 || a.K > 6144) return false;
   if (mode == 1 && epi != 2) return false;
