@@ -87,3 +87,82 @@ class KVCache:
         n = min(self.offset, n)
         self.offset -= n
         return n
+
+
+class SequenceSlots:
+    """Host-side table of the sequences a batched engine holds: ``length[s]`` is the number of tokens slot ``s`` has seen (the
+    position of its next token), ``-1`` marks a free slot.  One table is shared by the per-layer caches of a model, so a position
+    is advanced once per step, not once per layer.  Freed slots are handed out again lowest-first; the buffers behind a slot are
+    not cleared -- a reader may only touch what the new owner's positions cover."""
+
+    def __init__(self, n_slots: int = 1):
+        self.length: List[int] = [-1] * n_slots
+        self.listeners: List[Any] = []
+
+    @property
+    def n_slots(self) -> int:
+        return len(self.length)
+
+    def acquire(self) -> int:
+        for s, n in enumerate(self.length):
+            if n < 0:
+                self.length[s] = 0
+                return s
+        self.length.append(0)
+        for c in self.listeners:
+            c.grow(len(self.length))
+        return len(self.length) - 1
+
+    def release(self, slot: int) -> None:
+        if not (0 <= slot < len(self.length)) or self.length[slot] < 0:
+            raise ValueError(f"slot {slot} is not held")
+        self.length[slot] = -1
+
+    def live_tokens(self) -> int:
+        return sum(n for n in self.length if n > 0)
+
+
+class WindowKVCache:
+    """Keys / values of a sliding-window mixer for several sequences: one ring of ``window`` rows per slot, position ``p`` of a
+    sequence lives in row ``p % window`` (a token that has left every later query's window is the one overwritten).  Buffers are
+    token-major ``[slots, window, kv_heads * dim]`` so that a step's projection rows are appended as they are.  A step's own tokens
+    are NOT read from the ring (a long portion would overwrite rows its earlier queries still need): the mixer reads them from
+    the step's projection and appends after it has attended."""
+
+    def __init__(self, window: int, slots: Optional[SequenceSlots] = None):
+        self.window = int(window)
+        self.slots = slots if slots is not None else SequenceSlots(1)
+        self.slots.listeners.append(self)
+        self.keys = None
+        self.values = None
+
+    @property
+    def offset(self) -> int:                     # what generate_step reads: next position of the first sequence
+        return max(self.slots.length[0], 0)
+
+    def reserve(self, like_k: torch.Tensor, like_v: torch.Tensor) -> None:
+        if self.keys is None:
+            n = self.slots.n_slots
+            self.keys = torch.zeros((n, self.window, like_k.shape[-1]), dtype=like_k.dtype, device=like_k.device)
+            self.values = torch.zeros((n, self.window, like_v.shape[-1]), dtype=like_v.dtype, device=like_v.device)
+
+    def grow(self, n_slots: int) -> None:
+        if self.keys is not None and self.keys.shape[0] < n_slots:
+            n = max(n_slots, 2 * self.keys.shape[0])
+            for nm in ("keys", "values"):
+                old = getattr(self, nm)
+                new = torch.zeros((n,) + tuple(old.shape[1:]), dtype=old.dtype, device=old.device)
+                new[:old.shape[0]] = old
+                setattr(self, nm, new)
+
+    def append_rows(self, k: torch.Tensor, v: torch.Tensor, slot: int, pos0: int) -> None:
+        """Plain-torch append of one sequence's new rows (the HIP path appends a whole step in one launch)."""
+        n, w = k.shape[0], self.window
+        if n > w:
+            k, v, pos0, n = k[n - w:], v[n - w:], pos0 + n - w, w
+        rows = (torch.arange(pos0, pos0 + n, device=k.device) % w)
+        self.keys[slot, rows] = k
+        self.values[slot, rows] = v
+
+    def is_trimmable(self):
+        return False

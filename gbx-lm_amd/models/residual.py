@@ -1,0 +1,45 @@
+"""Residual updates that normalise the BRANCH, not the stream:  x <- x + mult * rms_norm(branch) * weight.
+
+The stream ``x`` is fp32 whatever the activation dtype is (it is a long sum of small terms); the branch arrives in the activation
+dtype, either as rows [T, W] or as ``top`` candidate rows per token [T, top, W] with fp32 mixing weights [T, top] (the routed
+experts' outputs: the weighted sum is folded in here, in fp32, so it is never rounded or stored).  Returns the activation-dtype
+image of the new stream, which is what the next sublayer reads.  GPU tensors: one launch (mixer_ops.residual_norm_add)."""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+from torch import nn
+
+
+class BranchNormResidual(nn.Module):
+    def __init__(self, width: int, eps: float, mult: float = 1.0):
+        super().__init__()
+        self.register_buffer("weight", torch.ones(width, dtype=torch.float32))
+        self.eps, self.mult = float(eps), float(mult)
+
+    def forward(self, x: torch.Tensor, branch: torch.Tensor, mix: Optional[torch.Tensor], act_dtype: torch.dtype) -> torch.Tensor:
+        """Updates ``x`` (fp32 [T, W]) in place and returns its image in ``act_dtype`` (x itself when that is fp32)."""
+        if x.is_cuda:
+            from .. import mixer_ops as M
+            return M.residual_norm_add(x, branch, mix, self.weight, self.eps, self.mult, act_dtype)
+        z = branch.float()
+        if mix is not None:
+            z = (z * mix.float().unsqueeze(-1)).sum(1)
+        x.add_(self.mult * z * torch.rsqrt(z.pow(2).mean(-1, keepdim=True) + self.eps) * self.weight.float())
+        return x if act_dtype == torch.float32 else x.to(act_dtype)
+
+
+class StreamRMSNorm(nn.Module):
+    """RMS norm of the fp32 stream into the activation dtype (the model's last norm)."""
+
+    def __init__(self, width: int, eps: float):
+        super().__init__()
+        self.register_buffer("weight", torch.ones(width, dtype=torch.float32))
+        self.eps = float(eps)
+
+    def forward(self, x: torch.Tensor, act_dtype: torch.dtype) -> torch.Tensor:
+        if x.is_cuda:
+            from .. import mixer_ops as M
+            return M.stream_rmsnorm(x, self.weight, self.eps, act_dtype)
+        return (x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + self.eps) * self.weight.float()).to(act_dtype)

@@ -115,3 +115,46 @@ class SwitchGLU(nn.Module):
             act = self.activation(x_up, x_gate)
         y = self.down_proj(act, indices)                            # [..., k, 1, D]
         return y.squeeze(-2)
+
+
+class DenseRoutedGLU(nn.Module):
+    """Top-k routed gated MLPs over unquantised stacked experts, rows of a ragged step in, the chosen experts' outputs out.
+
+    Router: logits in fp32 (``router`` is kept in fp32), probabilities = softmax over ALL experts, the ``top`` largest are chosen
+    (ties: the lower expert index); their mixing weights are those probabilities, divided by their sum only if ``renormalize``.
+    Expert e: down_e(silu(gate_e h) * (up_e h)); ``gate_up`` stacks gate_e over up_e as [E, 2F, K], ``down`` is [E, K, F].
+    ``forward`` returns (y [T, top, K], weights fp32 [T, top]): the weighted sum is left to the caller, which folds it into its
+    normalisation / residual launch."""
+
+    def __init__(self, input_dims: int, hidden_dims: int, num_experts: int, top: int, renormalize: bool = False):
+        super().__init__()
+        if not 1 <= top <= num_experts:
+            raise ValueError("top must lie in 1..num_experts")
+        self.input_dims, self.hidden_dims, self.num_experts, self.top, self.renormalize = input_dims, hidden_dims, num_experts, top, renormalize
+        self.register_buffer("router", torch.zeros((num_experts, input_dims), dtype=torch.float32))
+        self.register_buffer("gate_up", torch.zeros((num_experts, 2 * hidden_dims, input_dims)))
+        self.register_buffer("down", torch.zeros((num_experts, input_dims, hidden_dims)))
+
+    def route(self, h: torch.Tensor):
+        if h.is_cuda:
+            from .. import mixer_ops as M
+            return M.route_topk(h, self.router, self.top, self.renormalize)
+        probs = torch.softmax(F.linear(h.float(), self.router.float()), dim=-1)
+        w, idx = torch.topk(probs, self.top, dim=-1)
+        if self.renormalize:
+            w = w / w.sum(-1, keepdim=True)
+        return idx.to(torch.int32), w
+
+    def forward(self, h: torch.Tensor):
+        idx, w = self.route(h)
+        if h.is_cuda:
+            from .. import mixer_ops as M
+            return M.expert_glu(h, self.gate_up, self.down, idx), w
+        f = self.hidden_dims
+        y = torch.empty((h.shape[0], self.top, self.input_dims), dtype=h.dtype, device=h.device)
+        for e in range(self.num_experts):
+            t, s = torch.nonzero(idx == e, as_tuple=True)
+            if t.numel():
+                gu = F.linear(h[t], self.gate_up[e])
+                y[t, s] = F.linear(F.silu(gu[:, :f]) * gu[:, f:], self.down[e])
+        return y, w

@@ -18,7 +18,7 @@ from typing import Any, Callable, Generator, List, Optional, Tuple, Type, Union
 import torch
 from torch import nn
 
-from .models import qdeepseek_v3, qllama, qmixtral, qphi3, qqwen2, qqwen3, qqwen3_moe
+from .models import qdeepseek_v3, qllama, qmixtral, qphi3, qqwen2, qqwen3, qqwen3_moe, revitar
 from .models import cache as cache_mod
 from .models.quantized_linear_gba import QuantizedLinear
 from .tokenizer_utils import TokenizerWrapper, load_tokenizer
@@ -32,6 +32,7 @@ MODEL_MAPPING = {
     "qwen2": qqwen2,
     "qwen3": qqwen3,
     "qwen3_moe": qqwen3_moe,
+    "revitar": revitar,       # dense (unquantised) checkpoint; its config names itself by "architecture"
 }
 
 _DQ_KEYS = ('qstatistic', 'qscales_scales', 'qzeros_scales', 'qscales_zeros', 'qzeros_zeros')
@@ -61,7 +62,7 @@ class GenerationResponse:
 
 # --------------------------------------------------------------------------------------------- load
 def _get_classes(config: dict):
-    model_type = config["model_type"]
+    model_type = config["model_type"] if "model_type" in config else str(config.get("architecture", "")).lower()
     if model_type not in MODEL_MAPPING:
         msg = f"Model type {model_type} not supported."
         logging.error(msg)
@@ -155,11 +156,12 @@ def _reconcile_with_checkpoint(model, weights, use_double_quantization: bool, us
 def load_model(model_path: Path, lazy: bool = False, model_config: dict = {}, bits: int = 4, group_size: int = 64,
                is_conversion: bool = False,
                get_model_classes: Callable[[dict], Tuple[Type[nn.Module], Type]] = _get_classes,
-               device=None):
+               device=None, dtype: Optional[torch.dtype] = None):
     """Build the model from ``config.json`` + ``quant_strategy.json`` + ``model*.safetensors`` (utils.py:752-879).
 
     Returns ``(model, config)``.  ``lazy`` is accepted for signature parity; tensors are always materialised
-    on ``device`` (default: this rank's GPU if one is visible).
+    on ``device`` (default: this rank's GPU if one is visible).  ``dtype`` (dense checkpoints only) casts the matrices and the
+    embedding, e.g. ``torch.float32`` for a model stored in bf16 that is to run in true 32-bit.
     """
     from safetensors.torch import load_file
 
@@ -216,6 +218,20 @@ def load_model(model_path: Path, lazy: bool = False, model_config: dict = {}, bi
 
     if hasattr(model, "sanitize"):
         weights = model.sanitize(weights)
+
+    if not getattr(model_class, "quantized", True):       # dense checkpoint: every tensor must be there and must fit
+        if dtype is not None:
+            weights = {k: (v.to(dtype) if v.is_floating_point() and v.dtype != torch.float32 else v) for k, v in weights.items()}
+        have = {k for k, _ in model.named_parameters()} | {k for k, _ in model.named_buffers()}
+        missing = sorted(have - set(weights))
+        if missing:
+            raise ValueError(f"checkpoint lacks {len(missing)} tensors, e.g. {missing[:3]}")
+        skipped = load_weights(model, weights, device=device)
+        if skipped:
+            raise ValueError(f"checkpoint tensors without a place in the model: {skipped[:3]}")
+        model.to(device)
+        model.eval()
+        return model, config
 
     QuantizedLinear.reinit_module(model, **quantization, strategy=strategy,
                                   use_double_quantization=use_double_quantization, use_q_perm=use_q_perm)
