@@ -290,3 +290,69 @@ def check(rc: int) -> None:
     if rc == GBX_ERR_UNSUPPORTED:
         raise NotImplementedError(msg)
     raise RuntimeError(msg)
+
+
+# --------------------------------------------------------------------------- libgbx_mixers.so (include/gbx_mixers.h)
+_MSO = os.path.join(_CSRC, "libgbx_mixers.so")
+_mlib = None
+GBXM_BF16, GBXM_F32 = 1, 2
+
+
+class WindowAttnArgs(ctypes.Structure):
+    """Mirror of ``gbxm_window_attn_args``."""
+    _fields_ = [("qkv", ctypes.c_void_p), ("row_stride", ctypes.c_int64), ("kcache", ctypes.c_void_p), ("vcache", ctypes.c_void_p),
+                ("seq", ctypes.c_void_p), ("tok", ctypes.c_void_p), ("tiles", ctypes.c_void_p), ("out", ctypes.c_void_p),
+                ("dist_mul", ctypes.c_void_p), ("dist_rate", ctypes.c_void_p), ("gate_bias", ctypes.c_void_p),
+                ("T", ctypes.c_int64), ("B", ctypes.c_int32), ("n_tiles", ctypes.c_int32), ("q_tile", ctypes.c_int32),
+                ("H", ctypes.c_int32), ("G", ctypes.c_int32), ("dk", ctypes.c_int32), ("dv", ctypes.c_int32), ("window", ctypes.c_int32),
+                ("scale", ctypes.c_float), ("softcap", ctypes.c_float), ("decode_only", ctypes.c_int32), ("act", ctypes.c_int32)]
+
+
+def mixers_so_path() -> str:
+    return _MSO
+
+
+def build_mixers(force: bool = False, jobs: int = 8) -> str:
+    """Compile only libgbx_mixers.so (a handful of sources) in-tree."""
+    cmd = ["make", "-C", _CSRC, f"-j{jobs}", "libgbx_mixers.so"]
+    if force:
+        cmd.append("-B")
+    subprocess.check_call(cmd, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
+    return _MSO
+
+
+def mixers() -> ctypes.CDLL:
+    """The ragged-step kernel library; compiled on first use when the checkout holds no built copy.  No fallback: raises."""
+    global _mlib
+    if _mlib is None:
+        if not os.path.exists(_MSO):
+            build_mixers()
+        import torch
+        torch.cuda.is_available()                   # torch's HIP runtime first (see lib())
+        L = ctypes.CDLL(_MSO)
+        i64, i32, p, f32, sz = ctypes.c_int64, ctypes.c_int32, ctypes.c_void_p, ctypes.c_float, ctypes.c_size_t
+        L.gbxm_version.restype = ctypes.c_int
+        L.gbxm_last_error.restype = ctypes.c_char_p
+        L.gbxm_embed_scaled.argtypes = [p, p, p, p, i64, i32, f32, i32, p]
+        L.gbxm_segment_rmsnorm.argtypes = [p, i64, i64, i32, i32, p, p, f32, i32, p]
+        L.gbxm_residual_norm_add.argtypes = [p, p, p, p, p, i64, i32, i32, f32, f32, i32, p]
+        L.gbxm_stream_rmsnorm.argtypes = [p, p, p, i64, i32, f32, i32, p]
+        L.gbxm_route_topk.argtypes = [p, p, p, p, i64, i32, i32, i32, i32, i32, p]
+        L.gbxm_expert_glu_workspace.argtypes = [i64, i32, i32, i32, i32, i32]
+        L.gbxm_expert_glu_workspace.restype = sz
+        L.gbxm_expert_glu.argtypes = [p, p, p, p, p, i64, i32, i32, i32, i32, i32, p, sz, p]
+        L.gbxm_window_attention.argtypes = [ctypes.POINTER(WindowAttnArgs), p]
+        L.gbxm_window_append.argtypes = [p, i64, i32, i32, i32, p, p, p, p, i64, i32, i32, p]
+        _mlib = L
+    return _mlib
+
+
+def check_mixers(rc: int) -> None:
+    if rc == 0:
+        return
+    msg = mixers().gbxm_last_error().decode("utf-8", "replace")
+    if rc == GBX_ERR_INVALID:
+        raise ValueError(msg)
+    if rc == GBX_ERR_UNSUPPORTED:
+        raise NotImplementedError(msg)
+    raise RuntimeError(msg)

@@ -111,6 +111,11 @@ class Model(nn.Module):
     def layers(self):
         return self.model.layers
 
+    def required_kernels(self) -> None:
+        """Load (and, in a checkout without built files, first compile) the one kernel library this model runs on."""
+        from .. import _lib
+        _lib.mixers()
+
     def make_cache(self) -> List[Any]:
         """Per-layer caches over one shared slot table; slot 0 is handed to the one-sequence generate loop."""
         slots = SequenceSlots(1)

@@ -1,0 +1,74 @@
+/* C-ABI of libgbx_mixers.so: kernels of sequence mixers, routed feed-forwards and stream updates over RAGGED step batches
+ * (gfx950).  A step's rows lie back to back; two int32 tables describe them:
+ *   seq [B][4] = slot, position of the sequence's first new row, number of new rows, index of its first row in the step
+ *   tok [T][2] = sequence of the step the row belongs to, position of the row
+ * dtype codes: 1 = bf16, 2 = fp32 (activation dtype `act`; statistics, scores, gates and the stream are fp32 in both).
+ * Every function returns 0 or an error code (1 invalid argument, 2 HIP error, 3 unsupported shape: the caller picks another
+ * kernel) and leaves a text for gbxm_last_error().  All launches go to `stream`; nothing synchronises. */
+#pragma once
+#include <stddef.h>
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define GBXM_OK 0
+#define GBXM_ERR_INVALID 1
+#define GBXM_ERR_HIP 2
+#define GBXM_ERR_UNSUPPORTED 3
+#define GBXM_BF16 1
+#define GBXM_F32 2
+
+int gbxm_version(void);
+const char* gbxm_last_error(void);
+
+/* x[t] = table[token[t]] * scale (fp32 stream) and its image h in the activation dtype (h may be null when act is fp32). */
+int gbxm_embed_scaled(const void* table, const int64_t* tokens, float* x, void* h, int64_t T, int32_t width, float scale,
+                      int32_t act, void* stream);
+/* In place: rows[t][0:n0] and rows[t][n0:n0+n1] each RMS-normalised over the whole segment (fp32 statistics), times w0 / w1. */
+int gbxm_segment_rmsnorm(void* rows, int64_t T, int64_t row_stride, int32_t n0, int32_t n1, const float* w0, const float* w1,
+                         float eps, int32_t act, void* stream);
+/* x[t] += mult * rms_norm(z[t]) * w, z = branch[t] (top == 1, mix null) or sum_s mix[t][s] * branch[t][s]; h = image of x. */
+int gbxm_residual_norm_add(float* x, const void* branch, const float* mix, const float* w, void* h, int64_t T, int32_t width,
+                           int32_t top, float eps, float mult, int32_t act, void* stream);
+/* out[t] = rms_norm(x[t]) * w in the activation dtype. */
+int gbxm_stream_rmsnorm(const float* x, const float* w, void* out, int64_t T, int32_t width, float eps, int32_t act, void* stream);
+/* Router: logits = router (fp32 [E][K]) . h[t], probabilities over all E, the `top` largest (ties: lower index); weights are
+ * the probabilities, divided by their sum if renorm. */
+int gbxm_route_topk(const void* h, const float* router, int32_t* idx, float* weight, int64_t T, int32_t K, int32_t E, int32_t top,
+                    int32_t renorm, int32_t act, void* stream);
+/* y[t][s] = down[e] (silu(gate[e] h[t]) * (up[e] h[t])), e = idx[t][s]; gate_up [E][2F][K] (gate rows, then up rows),
+ * down [E][K][F].  `ws` (bytes from gbxm_expert_glu_workspace) lets prompt-sized steps run as grouped matrix-core products. */
+size_t gbxm_expert_glu_workspace(int64_t T, int32_t K, int32_t F, int32_t E, int32_t top, int32_t act);
+int gbxm_expert_glu(const void* h, const void* gate_up, const void* down, const int32_t* idx, void* y, int64_t T, int32_t K,
+                    int32_t F, int32_t E, int32_t top, int32_t act, void* ws, size_t ws_bytes, void* stream);
+
+/* Gated sliding-window attention (see gbx-lm_amd/models/window_attention.py for the equations).  qkv rows: q (H*dk) | k (G*dk) |
+ * v (G*dv), already normalised; ring caches [slots][window][G*dk] and [slots][window][G*dv] hold positions BEFORE the step. */
+typedef struct {
+  const void* qkv;
+  int64_t row_stride;           /* elements */
+  const void* kcache;
+  const void* vcache;
+  const int32_t* seq;           /* [B][4] */
+  const int32_t* tok;           /* [T][2] */
+  const int32_t* tiles;         /* [n_tiles][2]: sequence of the step, first row of the tile inside it (prompt kernel) */
+  void* out;                    /* [T][H*dv] */
+  const float* dist_mul;        /* [H] */
+  const float* dist_rate;       /* [H] */
+  const float* gate_bias;       /* [H] */
+  int64_t T;
+  int32_t B, n_tiles, q_tile;
+  int32_t H, G, dk, dv, window;
+  float scale, softcap;
+  int32_t decode_only;          /* every sequence brings one row */
+  int32_t act;
+} gbxm_window_attn_args;
+int gbxm_window_attention(const gbxm_window_attn_args* a, void* stream);
+/* Append the step's k / v rows to the rings (only the last `window` rows of a sequence are written). */
+int gbxm_window_append(const void* qkv, int64_t row_stride, int32_t nq, int32_t nk, int32_t nv, void* kcache, void* vcache,
+                       const int32_t* seq, const int32_t* tok, int64_t T, int32_t window, int32_t act, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
