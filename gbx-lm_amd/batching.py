@@ -34,7 +34,7 @@ class StepBatch:
         return all(n == 1 for n in self.n_new)
 
     @staticmethod
-    def build(slot: Sequence[int], pos0: Sequence[int], n_new: Sequence[int], device, q_tile: int = 64) -> "StepBatch":
+    def build(slot: Sequence[int], pos0: Sequence[int], n_new: Sequence[int], device, q_tile: int = 128) -> "StepBatch":
         rows, seq, tok, tiles = 0, [], [], []
         for b, (s, p, n) in enumerate(zip(slot, pos0, n_new)):
             if n <= 0:

@@ -140,7 +140,8 @@ class DenseRoutedGLU(nn.Module):
             from .. import mixer_ops as M
             return M.route_topk(h, self.router, self.top, self.renormalize)
         probs = torch.softmax(F.linear(h.float(), self.router.float()), dim=-1)
-        w, idx = torch.topk(probs, self.top, dim=-1)
+        w, idx = torch.sort(probs, dim=-1, descending=True, stable=True)      # of equal experts the lower index first
+        w, idx = w[..., :self.top], idx[..., :self.top]
         if self.renormalize:
             w = w / w.sum(-1, keepdim=True)
         return idx.to(torch.int32), w
