@@ -463,8 +463,84 @@ def prefill_leg(model, cfg, dev, B=8, T=4096):
                     "bf16 GEMMs on pre-expanded weights -- no dequantisation runs in that loop"}
 
 
+REVITAR_SIZES = {
+    # name: Revitar geometry, and the Qwen3-MoE (the closest existing family: grouped-query attention + routed experts) of equal size
+    "a3b-like": dict(width=2048, heads=32, kv_heads=4, dim=128, vdim=128, window=4096, experts=128, top=8, ff=768, n_layers=4, vocab=32000),
+    "small": dict(width=1024, heads=16, kv_heads=4, dim=64, vdim=64, window=1024, experts=16, top=2, ff=512, n_layers=4, vocab=32000),
+    "wide-heads": dict(width=4096, heads=32, kv_heads=8, dim=128, vdim=128, window=2048, experts=8, top=2, ff=2048, n_layers=2, vocab=32000),
+}
+
+
+def revitar_bench(args):
+    """``--design revitar``: prefill and decode throughput of Revitar at layer sizes of real models (random weights, bf16), beside
+    Qwen3-MoE of equal size on this framework (its experts and projections are GBA-packed at 4 bits: fewer weight bytes per token).
+    One JSON line; the default workload of this file is untouched."""
+    from gbx_lm_amd import synthetic as S
+    from gbx_lm_amd.batching import BatchScheduler
+    from gbx_lm_amd.models.cache import make_prompt_cache
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+
+    def clock(fn, reps):
+        fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / reps
+
+    out = {}
+    for name in args.sizes.split(","):
+        g = REVITAR_SIZES[name]
+        res = {"geometry": g}
+        model = S.build_revitar(S.revitar_config(**g), device=dev, seed=0)
+        toks = lambda n, o=0: [(o + i * 7919) % g["vocab"] for i in range(n)]
+        for T in (512, 4096):
+            def prefill():
+                eng = BatchScheduler(model)
+                eng.step([("p", toks(T))])
+            res[f"prefill_T{T}_tok_s"] = round(T / clock(prefill, 3) * 1e3)
+        for B in (1, 32):
+            eng = BatchScheduler(model)
+            ctx = min(g["window"], 2048)
+            eng.step([(i, toks(ctx, i)) for i in range(B)])
+            state = {"t": 0}
+            def decode():
+                state["t"] += 1
+                eng.step([(i, [(state["t"] * 31 + i) % g["vocab"]]) for i in range(B)])
+            res[f"decode_B{B}_ctx{ctx}_tok_s"] = round(B / clock(decode, args.steps if args.steps < 200 else 64) * 1e3)
+            del eng
+        del model
+        torch.cuda.empty_cache()
+        # the closest existing model at equal size
+        qcfg = dict(S.QWEN3_30B_A3B, hidden_size=g["width"], num_attention_heads=g["heads"], num_key_value_heads=g["kv_heads"], head_dim=g["dim"],
+                    num_experts=g["experts"], num_experts_per_tok=g["top"], moe_intermediate_size=g["ff"], num_hidden_layers=g["n_layers"],
+                    vocab_size=g["vocab"], mlp_only_layers=[], decoder_sparse_step=1)
+        qm = S.build_model(qcfg, S.make_strategy("S40", g["n_layers"], 128), device=dev, seed=0)
+        for T in (512, 4096):
+            ids = torch.tensor(toks(T), device=dev)[None]
+            def qprefill():
+                with torch.no_grad():
+                    qm(ids, cache=make_prompt_cache(qm))
+            res[f"qwen3moe_prefill_T{T}_tok_s"] = round(T / clock(qprefill, 3) * 1e3)
+        for B in (1, 32):
+            ctx = min(g["window"], 2048)
+            r = decode_leg(qm, qcfg, dev, B, min(ctx, 256), 64, 4)
+            res[f"qwen3moe_decode_B{B}_ctx256_tok_s"] = round(r["tok_s"])
+        del qm
+        torch.cuda.empty_cache()
+        out[name] = res
+    print(json.dumps({"metric": "revitar_throughput", "unit": "tokens/s", "dtype": "bf16", "data": "synthetic", "sizes": out}))
+
+
 def main():
     ap = argparse.ArgumentParser()
+    ap.add_argument("--design", default=None, choices=["revitar"], help="side benchmark of one model design beside the closest existing "
+                    "family at equal size (own JSON line; the default workload and its contract are unchanged)")
+    ap.add_argument("--sizes", default="small,a3b-like", help="--design revitar: comma-separated names of REVITAR_SIZES")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=512, help="timed decode steps (default: > 0.5 s of GPU time, so that a coarse GPU-busy sampler sees the run)")
     ap.add_argument("--warmup", type=int, default=8)
@@ -480,6 +556,10 @@ def main():
     ap.add_argument("--dry-run", action="store_true", help="CPU / gloo rehearsal of the multi-rank control flow")
     args = ap.parse_args()
 
+    if args.design == "revitar":
+        if not torch.cuda.is_available():
+            raise SystemExit("bench.py needs an MI355X")
+        return revitar_bench(args)
     if args.gpus > 1 and "WORLD_SIZE" not in os.environ:
         spawn_ranks(args.gpus)                                     # never returns; nothing has touched the GPU yet
     world = int(os.environ.get("WORLD_SIZE", "1"))

@@ -342,6 +342,7 @@ def mixers() -> ctypes.CDLL:
         L.gbxm_expert_glu_workspace.restype = sz
         L.gbxm_expert_glu.argtypes = [p, p, p, p, p, i64, i32, i32, i32, i32, i32, p, sz, p]
         L.gbxm_window_attention.argtypes = [ctypes.POINTER(WindowAttnArgs), p]
+        L.gbxm_window_attention_tiled.argtypes = [i32, i32, i32, i32]
         L.gbxm_window_append.argtypes = [p, i64, i32, i32, i32, p, p, p, p, i64, i32, i32, p]
         _mlib = L
     return _mlib

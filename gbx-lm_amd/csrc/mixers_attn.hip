@@ -98,10 +98,15 @@ __global__ __launch_bounds__(NT) void window_rows_kernel(const T* __restrict__ q
 }  // namespace
 
 int launch_window_tiles(const gbxm_window_attn_args& a, hipStream_t s);     // mixers_attn_mfma.hip; GBXM_ERR_UNSUPPORTED: not its shape
+bool window_tiles_shape(int dk, int dv);
 
 }  // namespace gbxm
 
 using namespace gbxm;
+
+extern "C" int gbxm_window_attention_tiled(int32_t dk, int32_t dv, int32_t act, int32_t decode_only) {
+  return act == GBXM_BF16 && !decode_only && window_tiles_shape(dk, dv);
+}
 
 extern "C" int gbxm_window_attention(const gbxm_window_attn_args* a, void* stream) {
   if (!a || !a->qkv || !a->kcache || !a->vcache || !a->seq || !a->tok || !a->out || !a->dist_mul || !a->dist_rate || !a->gate_bias)

@@ -139,7 +139,15 @@ int launch(const TileArgs& t, int n_tiles, int H, hipStream_t s) {
 
 }  // namespace
 
+bool window_tiles_shape(int dk, int dv) {
+  const int ok[][2] = {{64, 64}, {96, 64}, {128, 64}, {64, 128}, {128, 128}, {192, 128}, {256, 256}, {96, 96}, {64, 32}, {32, 32}, {32, 64}};
+  for (const auto& p : ok)
+    if (p[0] == dk && p[1] == dv) return true;
+  return false;
+}
+
 int launch_window_tiles(const gbxm_window_attn_args& a, hipStream_t s) {
+  if (!window_tiles_shape(a.dk, a.dv)) return GBXM_ERR_UNSUPPORTED;
   if (a.q_tile != 128 || a.H > 65535 || a.row_stride % 8 || (reinterpret_cast<uintptr_t>(a.qkv) | reinterpret_cast<uintptr_t>(a.kcache) |
                                                              reinterpret_cast<uintptr_t>(a.vcache) | reinterpret_cast<uintptr_t>(a.out)) % 16)
     return GBXM_ERR_UNSUPPORTED;

@@ -244,3 +244,50 @@ def write_checkpoint(path: str, config: Dict, strategy: Optional[Dict], seed: in
     save_file(sd, os.path.join(path, "model.safetensors"))
     write_tokenizer(path, config["vocab_size"], config.get("eos_token_id", config["vocab_size"] - 1))
     return model
+
+
+# ------------------------------------------------------------------------------------------------ Revitar (dense, ragged steps)
+def revitar_config(width: int, heads: int, kv_heads: int, dim: int, vdim: int, window: int, experts: int, top: int, ff: int,
+                   n_layers: int, vocab: int = 32000, softcap: float = 50.0, residual_mult: float = 0.3, embed_scale: float = 1.0) -> Dict:
+    """config.json of a Revitar model whose layers are all alike (benchmarks; a checkpoint may mix layers freely)."""
+    layer = {"type": "attention",
+             "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "mask": {"size": window},
+                       "scale": dim ** -0.5, "softcap": softcap},
+             "mlp": {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top}}}
+    return {"architecture": "Revitar", "vocab": vocab, "width": width, "layers": [dict(layer) for _ in range(n_layers)],
+            "norm": {"eps": 1e-6}, "residual_mult": residual_mult, "embedding": {"scale": embed_scale}}
+
+
+def build_revitar(config: Dict, device="cpu", seed: int = 0, act_dtype=torch.bfloat16):
+    """Random-init Revitar with real shapes, generated directly on ``device`` (no files)."""
+    from .models import revitar
+    device = torch.device(device)
+    args = revitar.ModelArgs.from_dict(config)
+    with torch.device("meta"):
+        model = revitar.Model(args)
+    model = model.to_empty(device=device)
+    gen = torch.Generator(device=device)
+    gen.manual_seed(seed)
+
+    def rnd(shape, std, dtype):
+        return (torch.randn(tuple(shape), device=device, generator=gen) * std).to(dtype)
+
+    for name, p in list(model.named_parameters()):
+        mod, _, attr = name.rpartition(".")
+        std = 1.0 if "embed_tokens" in name else p.shape[-1] ** -0.5
+        dict(model.named_modules())[mod]._parameters[attr] = torch.nn.Parameter(rnd(p.shape, std, act_dtype), requires_grad=False)
+    for name, b in list(model.named_buffers()):
+        mod, _, attr = name.rpartition(".")
+        m = dict(model.named_modules())[mod]
+        if attr in ("gate_up", "down"):
+            m._buffers[attr] = rnd(b.shape, b.shape[-1] ** -0.5, act_dtype)
+        elif attr == "router":
+            m._buffers[attr] = rnd(b.shape, 4.0 * b.shape[-1] ** -0.5, torch.float32)
+        elif attr in ("dist_mul", "dist_rate"):
+            m._buffers[attr] = torch.rand(tuple(b.shape), device=device, generator=gen) * 0.5 + 0.05
+        elif attr == "gate_bias":
+            m._buffers[attr] = torch.rand(tuple(b.shape), device=device, generator=gen) * 2.0 - 3.0
+        else:                                      # norm weights
+            m._buffers[attr] = torch.ones(tuple(b.shape), dtype=torch.float32, device=device)
+    model.eval()
+    return model

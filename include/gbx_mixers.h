@@ -65,6 +65,8 @@ typedef struct {
   int32_t act;
 } gbxm_window_attn_args;
 int gbxm_window_attention(const gbxm_window_attn_args* a, void* stream);
+/* 1 if a step of this kind runs on the matrix-core tile kernel, 0 if on the row kernel (tests and benchmarks name the kernel). */
+int gbxm_window_attention_tiled(int32_t dk, int32_t dv, int32_t act, int32_t decode_only);
 /* Append the step's k / v rows to the rings (only the last `window` rows of a sequence are written). */
 int gbxm_window_append(const void* qkv, int64_t row_stride, int32_t nq, int32_t nk, int32_t nv, void* kcache, void* vcache,
                        const int32_t* seq, const int32_t* tok, int64_t T, int32_t window, int32_t act, void* stream);

@@ -293,6 +293,48 @@ def test_router_mechanism(device):
 
 
 @pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows,k,f,experts,top", [(5, 64, 32, 6, 2), (300, 64, 96, 5, 3), (200, 160, 32, 3, 2), (40, 48, 20, 4, 1)])
+def test_expert_mechanism(device, dtype, rows, k, f, experts, top):
+    """Routed gated MLPs with GIVEN choices (so rounding cannot change them): few rows (one workgroup per row and choice), many rows
+    (grouped products, some experts unused, one expert with more than a tile of rows), sizes off the tile grid."""
+    from gbx_lm_amd.models.switch_layers import DenseRoutedGLU
+    g = torch.Generator().manual_seed(rows)
+    m = DenseRoutedGLU(k, f, experts, top)
+    m.gate_up.copy_(torch.randn((experts, 2 * f, k), generator=g) / math.sqrt(k))
+    m.down.copy_(torch.randn((experts, k, f), generator=g) / math.sqrt(f))
+    m.to(device)
+    m._buffers["gate_up"], m._buffers["down"] = m.gate_up.to(dtype), m.down.to(dtype)
+    h = torch.randn((rows, k), generator=g).to(dtype)
+    idx = torch.stack([torch.randperm(experts - 1, generator=g)[:top] for _ in range(rows)]).to(torch.int32)   # the last expert stays unused
+    idx[: rows // 2, 0] = 0 if top == 1 else idx[: rows // 2, 0]
+    if device == "cuda":
+        from gbx_lm_amd import mixer_ops as M, _lib
+        grouped = _lib.mixers().gbxm_expert_glu_workspace(rows, k, f, experts, top, _lib.GBXM_BF16 if dtype == torch.bfloat16 else _lib.GBXM_F32) > 0
+        assert grouped == (dtype == torch.bfloat16 and rows * top >= 256 and k % 32 == 0 and f % 32 == 0)
+        y = M.expert_glu(h.to(device), m.gate_up, m.down, idx.to(device))
+    else:
+        m.route = lambda _h: (idx, torch.ones((rows, top)))
+        y, _ = m(h)
+    gu, dn, hd = m.gate_up.cpu().to(O.F64), m.down.cpu().to(O.F64), h.to(O.F64)
+    for t in range(0, rows, max(1, rows // 25)):
+        for s_ in range(top):
+            e = int(idx[t, s_])
+            z = gu[e, :f] @ hd[t]
+            ref = dn[e] @ (z / (1 + torch.exp(-z)) * (gu[e, f:] @ hd[t]))
+            assert O.rel_err(y[t, s_][None], ref[None]) < (1e-5 if dtype == torch.float32 else 2e-2), (t, s_, e)
+
+
+@pytest.mark.gpu
+def test_prompt_portions_run_on_the_matrix_cores():
+    from gbx_lm_amd import _lib
+    L = _lib.mixers()
+    assert L.gbxm_window_attention_tiled(64, 128, _lib.GBXM_BF16, 0) == 1 and L.gbxm_window_attention_tiled(32, 32, _lib.GBXM_BF16, 0) == 1
+    assert L.gbxm_window_attention_tiled(64, 128, _lib.GBXM_BF16, 1) == 0 and L.gbxm_window_attention_tiled(64, 128, _lib.GBXM_F32, 0) == 0
+    assert L.gbxm_window_attention_tiled(24, 8, _lib.GBXM_BF16, 0) == 0
+
+
+@pytest.mark.parametrize("device", DEVICES)
 def test_greedy_generation_through_the_entry_points(checkpoints, device):
     """generate_step (the one-sequence loop) and BatchScheduler.generate (several prompts, ragged) produce the oracle's greedy
     continuation; a stop token ends one request while the others go on."""
