@@ -503,15 +503,18 @@ def revitar_bench(args):
                 eng = BatchScheduler(model)
                 eng.step([("p", toks(T))])
             res[f"prefill_T{T}_tok_s"] = round(T / clock(prefill, 3) * 1e3)
+            print(name, res, file=sys.stderr, flush=True)
+        ctx_of = {1: min(g["window"], 2048), 32: 256}
         for B in (1, 32):
             eng = BatchScheduler(model)
-            ctx = min(g["window"], 2048)
+            ctx = ctx_of[B]
             eng.step([(i, toks(ctx, i)) for i in range(B)])
             state = {"t": 0}
             def decode():
                 state["t"] += 1
                 eng.step([(i, [(state["t"] * 31 + i) % g["vocab"]]) for i in range(B)])
-            res[f"decode_B{B}_ctx{ctx}_tok_s"] = round(B / clock(decode, args.steps if args.steps < 200 else 64) * 1e3)
+            res[f"decode_B{B}_ctx{ctx}_tok_s"] = round(B / clock(decode, 64) * 1e3)
+            print(name, res, file=sys.stderr, flush=True)
             del eng
         del model
         torch.cuda.empty_cache()
@@ -527,9 +530,25 @@ def revitar_bench(args):
                     qm(ids, cache=make_prompt_cache(qm))
             res[f"qwen3moe_prefill_T{T}_tok_s"] = round(T / clock(qprefill, 3) * 1e3)
         for B in (1, 32):
-            ctx = min(g["window"], 2048)
-            r = decode_leg(qm, qcfg, dev, B, min(ctx, 256), 64, 4)
-            res[f"qwen3moe_decode_B{B}_ctx256_tok_s"] = round(r["tok_s"])
+            ctx = ctx_of[B]
+            if B == 1:                                   # the generate loop's path: prompt pass, then the graph-replayed single-token step
+                cache = make_prompt_cache(qm)
+                with torch.no_grad():
+                    y = torch.argmax(qm(torch.tensor(toks(ctx), device=dev)[None], cache=cache)[:, -1], -1)
+                state = {"y": y}
+                def qdecode():
+                    with torch.no_grad():
+                        state["y"] = torch.argmax(qm.decode_step(state["y"], cache), -1)
+            else:                                        # a synchronous batch through the model's own forward (eager launches)
+                cache = make_prompt_cache(qm)
+                ids = torch.tensor([toks(ctx, i) for i in range(B)], device=dev)
+                with torch.no_grad():
+                    y = torch.argmax(qm(ids, cache=cache)[:, -1], -1)
+                state = {"y": y}
+                def qdecode():
+                    with torch.no_grad():
+                        state["y"] = torch.argmax(qm(state["y"][:, None], cache=cache)[:, -1], -1)
+            res[f"qwen3moe_decode_B{B}_ctx{ctx}_tok_s"] = round(B / clock(qdecode, 64) * 1e3)
         del qm
         torch.cuda.empty_cache()
         out[name] = res

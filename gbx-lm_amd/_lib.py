@@ -305,7 +305,8 @@ class WindowAttnArgs(ctypes.Structure):
                 ("dist_mul", ctypes.c_void_p), ("dist_rate", ctypes.c_void_p), ("gate_bias", ctypes.c_void_p),
                 ("T", ctypes.c_int64), ("B", ctypes.c_int32), ("n_tiles", ctypes.c_int32), ("q_tile", ctypes.c_int32),
                 ("H", ctypes.c_int32), ("G", ctypes.c_int32), ("dk", ctypes.c_int32), ("dv", ctypes.c_int32), ("window", ctypes.c_int32),
-                ("scale", ctypes.c_float), ("softcap", ctypes.c_float), ("decode_only", ctypes.c_int32), ("act", ctypes.c_int32)]
+                ("scale", ctypes.c_float), ("softcap", ctypes.c_float), ("decode_only", ctypes.c_int32), ("act", ctypes.c_int32),
+                ("partial", ctypes.c_void_p), ("partial_splits", ctypes.c_int32)]
 
 
 def mixers_so_path() -> str:
@@ -337,9 +338,10 @@ def mixers() -> ctypes.CDLL:
         L.gbxm_segment_rmsnorm.argtypes = [p, i64, i64, i32, i32, p, p, f32, i32, p]
         L.gbxm_residual_norm_add.argtypes = [p, p, p, p, p, i64, i32, i32, f32, f32, i32, p]
         L.gbxm_stream_rmsnorm.argtypes = [p, p, p, i64, i32, f32, i32, p]
-        L.gbxm_route_topk.argtypes = [p, p, p, p, i64, i32, i32, i32, i32, i32, p]
+        L.gbxm_route_topk.argtypes = [p, p, p, i64, i32, i32, i32, p]
         L.gbxm_expert_glu_workspace.argtypes = [i64, i32, i32, i32, i32, i32]
         L.gbxm_expert_glu_workspace.restype = sz
+        L.gbxm_expert_glu_grouped.argtypes = [i64, i32, i32, i32, i32, i32]
         L.gbxm_expert_glu.argtypes = [p, p, p, p, p, i64, i32, i32, i32, i32, i32, p, sz, p]
         L.gbxm_window_attention.argtypes = [ctypes.POINTER(WindowAttnArgs), p]
         L.gbxm_window_attention_tiled.argtypes = [i32, i32, i32, i32]

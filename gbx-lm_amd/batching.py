@@ -16,6 +16,8 @@ from typing import Callable, Dict, Iterable, List, Optional, Sequence, Tuple
 
 import torch
 
+from . import env
+
 
 @dataclass
 class StepBatch:
@@ -52,6 +54,56 @@ class StepBatch:
                          packed[4 * nb:4 * nb + 2 * nt].view(nt, 2), q_tile, packed[4 * nb + 2 * nt:].view(-1, 2))
 
 
+class _DecodeGraph:
+    """One decode step (every sequence brings one token) of a fixed set of slots, captured in a HIP graph.  Tokens and the step's
+    descriptor tables live in one static device buffer that a single host-to-device copy refreshes before each replay; the
+    launches, their grids and every pointer they read are the same from step to step, only positions and tokens change."""
+
+    def __init__(self, sched: "BatchScheduler", slots: Tuple[int, ...]):
+        self.slots = slots
+        b = len(slots)
+        dev = sched.device
+        # int64 words: tokens [b] | seq [b, 4] as int32 pairs | tok [b, 2] | tiles [b, 2]
+        self.words = b + 2 * b + b + b
+        self.static = torch.zeros((self.words,), dtype=torch.int64, device=dev)
+        self.pinned = [torch.zeros((self.words,), dtype=torch.int64, pin_memory=True) for _ in range(2)]
+        self.copied = [None, None]
+        self.turn = 0
+        i32 = self.static.view(torch.int32)
+        self.tokens = self.static[:b]
+        self.batch = StepBatch(list(slots), [0] * b, [1] * b, b, i32[2 * b:6 * b].view(b, 4), i32[6 * b:8 * b].view(b, 2), 128,
+                               i32[8 * b:10 * b].view(b, 2))
+        self.graph = None
+        self.logits = None
+
+    def fill(self, tokens: Sequence[int], pos0: Sequence[int]) -> None:
+        k = self.turn % 2
+        self.turn += 1
+        if self.copied[k] is not None:
+            self.copied[k].synchronize()                 # the copy that last read this host buffer has run
+        host = self.pinned[k]
+        b = len(self.slots)
+        host[:b] = torch.tensor(tokens, dtype=torch.int64)
+        i32 = host.view(torch.int32)
+        i32[2 * b:6 * b] = torch.tensor([v for i, (s, p) in enumerate(zip(self.slots, pos0)) for v in (s, p, 1, i)], dtype=torch.int32)
+        i32[6 * b:8 * b] = torch.tensor([v for i, p in enumerate(pos0) for v in (i, p)], dtype=torch.int32)
+        i32[8 * b:10 * b] = torch.tensor([v for i in range(b) for v in (i, 0)], dtype=torch.int32)
+        self.static.copy_(host, non_blocking=True)
+        self.copied[k] = torch.cuda.Event()
+        self.copied[k].record(torch.cuda.current_stream(self.static.device))
+        self.batch.pos0 = list(pos0)
+
+    def run(self, sched: "BatchScheduler") -> torch.Tensor:
+        if self.graph is None:
+            torch.cuda.synchronize(sched.device)
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                self.logits = sched.model.logits(sched.model.forward_tokens(self.tokens, self.batch, sched.caches))
+            self.graph = g
+        self.graph.replay()
+        return self.logits
+
+
 class BatchScheduler:
     """Sequences in slots, stepped together.  ``step`` takes what each live sequence brings next and returns the logits of the rows
     that are asked for; ``release`` gives a finished sequence's slot back.  ``max_tokens`` bounds the tokens live sequences may hold
@@ -65,6 +117,11 @@ class BatchScheduler:
         self.max_tokens = max_tokens
         self.slot_of: Dict[object, int] = {}
         self.device = next(model.parameters()).device
+        # decode-only steps of a set of slots that keeps coming back are replayed from a HIP graph (captured at its third step)
+        self.use_graphs = self.device.type == "cuda" and env.flag("GBX_STEP_GRAPH")
+        self._graphs: Dict[Tuple[int, ...], _DecodeGraph] = {}
+        self._seen: Dict[Tuple[int, ...], int] = {}
+        self._buffers = None
 
     def position(self, seq_id) -> int:
         return self.slots.length[self.slot_of[seq_id]]
@@ -90,6 +147,17 @@ class BatchScheduler:
         slot = [self.slot_of[i] for i, _ in entries]
         pos0 = [self.slots.length[s] for s in slot]
         n_new = [len(t) for _, t in entries]
+        if self.use_graphs and all(n == 1 for n in n_new) and len(slot) <= 256:
+            logits = self._graph_step(tuple(slot), [ts[0] for _, ts in entries], pos0)
+            if logits is not None:
+                for s in slot:
+                    self.slots.length[s] += 1
+                rows = [i for i in range(len(slot)) if want is None or len(want[i])]
+                if any(p != 0 for i in rows if want is not None for p in want[i]):
+                    raise ValueError("a wanted place lies outside the entry's tokens")
+                if not rows:
+                    return torch.empty((0, self.model.args.vocab), dtype=torch.float32, device=self.device)
+                return logits.index_select(0, torch.tensor(rows, dtype=torch.long, device=self.device)).float()
         batch = StepBatch.build(slot, pos0, n_new, self.device)
         tokens = torch.tensor([t for _, ts in entries for t in ts], dtype=torch.long)
         if self.device.type == "cuda":
@@ -109,6 +177,27 @@ class BatchScheduler:
             return torch.empty((0, self.model.args.vocab), dtype=torch.float32, device=self.device)
         idx = torch.tensor(rows, dtype=torch.long, device=self.device)
         return self.model.logits(hidden.index_select(0, idx)).float()
+
+    def _graph_step(self, slots: Tuple[int, ...], tokens: Sequence[int], pos0: Sequence[int]) -> Optional[torch.Tensor]:
+        """Replay (or, at the third step of this set of slots, capture) the decode graph; None: run the step eagerly."""
+        buffers = tuple(c.keys.data_ptr() if c.keys is not None else 0 for c in self.caches)
+        if buffers != self._buffers:                     # rings were (re)allocated: every captured pointer is stale
+            self._graphs.clear()
+            self._seen.clear()
+            self._buffers = buffers
+        if 0 in buffers:
+            return None
+        g = self._graphs.get(slots)
+        if g is None:
+            self._seen[slots] = self._seen.get(slots, 0) + 1
+            if self._seen[slots] < 3:
+                return None
+            if len(self._graphs) >= 8:                   # a few live compositions at most: drop the oldest
+                self._graphs.pop(next(iter(self._graphs)))
+            g = self._graphs[slots] = _DecodeGraph(self, slots)
+            self._seen.pop(slots, None)
+        g.fill(tokens, pos0)
+        return g.run(self)
 
     @torch.no_grad()
     def generate(self, prompts: Sequence[Sequence[int]], max_tokens: int = 64,

@@ -6,9 +6,12 @@
 //
 // Two kernels:
 //   * window_rows_kernel  -- any head sizes, fp32 or bf16: one workgroup per (row, kv head) takes all query heads of the group,
-//     scores by vector FMAs over a 64-key tile, then the value sum with the lanes across the value channels.  The kernel of decode
-//     steps (one row per sequence) and of every shape the matrix-core kernel does not take; all arithmetic fp32.
+//     scores by vector FMAs over a 64-key tile (16-byte key loads), then the value sum with the lanes across the value channels.  The
+//     kernel of decode steps (one row per sequence) and of every shape the matrix-core kernel does not take; all arithmetic fp32.
+//     A step of few rows splits each row's key tiles over several workgroups (fp32 partial sums, added in a fixed order by
+//     window_reduce_kernel), so that one sequence's decode step still reads its window with the whole chip.
 //   * window_tile_kernel  -- bf16 prompt portions on the matrix cores (second part of this file).
+#include <algorithm>
 #include "mixers_common.h"
 
 namespace gbxm {
@@ -16,7 +19,6 @@ namespace {
 
 constexpr int NT = 256;
 constexpr int KT = 64;            // keys per tile of the row kernel
-constexpr int MAXACC = 8;         // value sums a thread of the row kernel can own
 
 struct Geo {
   int H, G, dk, dv, window, nq, nk;
@@ -31,38 +33,82 @@ __device__ __forceinline__ const T* key_row(const T* qkv, int64_t stride, const 
                   : qkv + (row0 + (j - pos0)) * stride + seg_off;
 }
 
-template <typename T, bool FAST>
+// <q, k> over dk channels: q in LDS (fp32), k a global row.  VEC: 16-byte loads (dk a multiple of the vector, row 16-byte aligned).
+template <typename T, bool VEC>
+__device__ __forceinline__ float qk_dot(const float* __restrict__ q, const T* __restrict__ k, int dk) {
+  float dot = 0.f;
+  if constexpr (VEC) {
+    constexpr int PER = 16 / sizeof(T);
+    for (int d = 0; d < dk; d += PER) {
+      const uint4 raw = *reinterpret_cast<const uint4*>(k + d);
+      if constexpr (sizeof(T) == 2) {
+        const unsigned u[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          dot += q[d + 2 * i] * __uint_as_float(u[i] << 16);
+          dot += q[d + 2 * i + 1] * __uint_as_float(u[i] & 0xFFFF0000u);
+        }
+      } else {
+        dot += q[d] * __uint_as_float(raw.x) + q[d + 1] * __uint_as_float(raw.y) + q[d + 2] * __uint_as_float(raw.z) + q[d + 3] * __uint_as_float(raw.w);
+      }
+    }
+  } else {
+    for (int d = 0; d < dk; ++d) dot += q[d] * to_f32(k[d]);
+  }
+  return dot;
+}
+
+constexpr int RC = 8;             // query heads a workgroup of the row kernel takes at most
+constexpr int DCH = 128;          // value channels per lane pass (two per lane)
+constexpr int NCH = 4;            // lane passes: value sizes up to NCH * DCH
+
+// One workgroup = one row x one kv head x up to RC of its query heads x its share of the key tiles.
+//   scores: a thread per (head, key) of a 64-key tile, 16-byte key loads against the query in LDS, gates to LDS;
+//   values: a wave per key, lanes across the value channels (two each), every loaded value feeds all heads' sums;
+//   the four waves' sums meet in LDS in a fixed order.
+template <typename T, bool FAST, bool VEC>
 __global__ __launch_bounds__(NT) void window_rows_kernel(const T* __restrict__ qkv, int64_t stride, const T* __restrict__ kc, const T* __restrict__ vc,
                                                         const int* __restrict__ seq, const int* __restrict__ tok, T* __restrict__ out,
                                                         const float* __restrict__ dmul, const float* __restrict__ drate,
-                                                        const float* __restrict__ gbias, Geo g, int rc) {
-  extern __shared__ float lds[];                    // q [rc][dk] | gates [rc][KT]
+                                                        const float* __restrict__ gbias, Geo g, int rc, int splits, float* __restrict__ partial) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  const T** kptr = reinterpret_cast<const T**>(lds_raw);            // [KT] rows of the tile's keys
+  const T** vptr = kptr + KT;                                        // [KT] and values
+  float* ql = reinterpret_cast<float*>(vptr + KT);                   // [rc][dk]
+  float* gl = ql + rc * g.dk;                                        // [rc][KT]
+  float* sums = gl + rc * KT;                                        // [NW][rc * dv]
+  constexpr int NW = NT / 64;
   const int64_t t = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int R = g.H / g.G;
   const int chunks = (R + rc - 1) / rc;
   const int kvh = blockIdx.y / chunks, r0 = (blockIdx.y % chunks) * rc;
   const int nr = min(rc, R - r0);                   // query heads of this workgroup: kvh * R + r0 + (0 .. nr-1)
-  float* ql = lds;
-  float* gl = lds + rc * g.dk;
   const int b = tok[2 * t], pos = tok[2 * t + 1];
   const int slot = seq[4 * b], pos0 = seq[4 * b + 1], row0 = seq[4 * b + 3];
   const int nkv_k = g.G * g.dk, nkv_v = g.G * g.dv;
   const T* qrow = qkv + t * stride + (kvh * R + r0) * g.dk;
   for (int i = threadIdx.x; i < nr * g.dk; i += NT) ql[i] = to_f32(qrow[i]);
-  float acc[MAXACC];
+  float acc[NCH][RC][2];
 #pragma unroll
-  for (int i = 0; i < MAXACC; ++i) acc[i] = 0.f;
+  for (int c = 0; c < NCH; ++c)
+#pragma unroll
+    for (int r = 0; r < RC; ++r) acc[c][r][0] = acc[c][r][1] = 0.f;
+  const bool pair_loads = g.dv % 2 == 0 && VEC;     // (VEC: rows are 16-byte aligned, so channel pairs are 4-byte aligned)
   const int jlo = max(0, pos - g.window + 1);
-  for (int jt = jlo; jt <= pos; jt += KT) {
-    __syncthreads();                                // q ready; gates of the previous tile consumed
+  for (int jt = jlo + static_cast<int>(blockIdx.z) * KT; jt <= pos; jt += KT * splits) {     // this workgroup's share of the key tiles
+    __syncthreads();                                // the previous tile's gates and rows have been consumed
+    if (threadIdx.x < KT) {
+      const int j = min(jt + static_cast<int>(threadIdx.x), pos);
+      kptr[threadIdx.x] = key_row(qkv, stride, kc, nkv_k, g.nq, slot, pos0, row0, g.window, j) + kvh * g.dk;
+      vptr[threadIdx.x] = key_row(qkv, stride, vc, nkv_v, g.nq + g.nk, slot, pos0, row0, g.window, j) + kvh * g.dv;
+    }
+    __syncthreads();
     for (int i = threadIdx.x; i < nr * KT; i += NT) {
-      const int r = i / KT, j = jt + i % KT;
+      const int r = i / KT, jj = i % KT, j = jt + jj;
       float gate = 0.f;
       if (j <= pos) {
-        const T* kr = key_row(qkv, stride, kc, nkv_k, g.nq, slot, pos0, row0, g.window, j) + kvh * g.dk;
-        const float* qr = ql + r * g.dk;
-        float dot = 0.f;
-        for (int d = 0; d < g.dk; ++d) dot += qr[d] * to_f32(kr[d]);
+        const float dot = qk_dot<T, VEC>(ql + r * g.dk, kptr[jj], g.dk);
         const int head = kvh * R + r0 + r;
         float s = dot * g.scale;
         if (g.softcap > 0.f) s = g.softcap * tanh_<FAST>(s / g.softcap);
@@ -73,26 +119,98 @@ __global__ __launch_bounds__(NT) void window_rows_kernel(const T* __restrict__ q
     }
     __syncthreads();
     const int nj = min(KT, pos - jt + 1);
+#pragma unroll 4
+    for (int jj = wave; jj < nj; jj += NW) {
+      const T* vr = vptr[jj];
 #pragma unroll
-    for (int a = 0; a < MAXACC; ++a) {
-      const int i = threadIdx.x + a * NT;
-      if (i < nr * g.dv) {
-        const int r = i / g.dv, d = i % g.dv;
-        float s = acc[a];
-        for (int jj = 0; jj < nj; ++jj) {
-          const T* vr = key_row(qkv, stride, vc, nkv_v, g.nq + g.nk, slot, pos0, row0, g.window, jt + jj) + kvh * g.dv;
-          s += gl[r * KT + jj] * to_f32(vr[d]);
+      for (int c = 0; c < NCH; ++c) {
+        const int d0 = c * DCH + 2 * lane;
+        if (d0 < g.dv) {
+          float v0, v1 = 0.f;
+          if (pair_loads) {
+            if constexpr (sizeof(T) == 2) {
+              const unsigned u = *reinterpret_cast<const unsigned*>(vr + d0);
+              v0 = __uint_as_float(u << 16); v1 = __uint_as_float(u & 0xFFFF0000u);
+            } else {
+              const float2 f = *reinterpret_cast<const float2*>(vr + d0);
+              v0 = f.x; v1 = f.y;
+            }
+          } else {
+            v0 = to_f32(vr[d0]);
+            if (d0 + 1 < g.dv) v1 = to_f32(vr[d0 + 1]);
+          }
+#pragma unroll
+          for (int r = 0; r < RC; ++r)
+            if (r < nr) {
+              const float gate = gl[r * KT + jj];
+              acc[c][r][0] += gate * v0;
+              acc[c][r][1] += gate * v1;
+            }
         }
-        acc[a] = s;
       }
     }
   }
-  T* orow = out + t * (static_cast<int64_t>(g.H) * g.dv) + (kvh * R + r0) * g.dv;
+  __syncthreads();
 #pragma unroll
-  for (int a = 0; a < MAXACC; ++a) {
-    const int i = threadIdx.x + a * NT;
-    if (i < nr * g.dv) orow[i] = from_f32<T>(acc[a]);
+  for (int c = 0; c < NCH; ++c) {
+    const int d0 = c * DCH + 2 * lane;
+    if (d0 < g.dv)
+#pragma unroll
+      for (int r = 0; r < RC; ++r)
+        if (r < nr) {
+          sums[(wave * rc + r) * g.dv + d0] = acc[c][r][0];
+          if (d0 + 1 < g.dv) sums[(wave * rc + r) * g.dv + d0 + 1] = acc[c][r][1];
+        }
   }
+  __syncthreads();
+  const int64_t hv = static_cast<int64_t>(g.H) * g.dv;
+  float* prow = splits > 1 ? partial + (static_cast<int64_t>(blockIdx.z) * gridDim.x + t) * hv + (kvh * R + r0) * g.dv : nullptr;
+  T* orow = out + t * hv + (kvh * R + r0) * g.dv;
+  for (int i = threadIdx.x; i < nr * g.dv; i += NT) {
+    float s = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) s += sums[w * rc * g.dv + i];
+    if (prow) prow[i] = s; else orow[i] = from_f32<T>(s);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(NT) void window_reduce_kernel(const float* __restrict__ partial, T* __restrict__ out, int64_t n, int splits) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * NT + threadIdx.x;
+  if (i >= n) return;
+  float s = 0.f;
+  for (int z = 0; z < splits; ++z) s += partial[z * n + i];
+  out[i] = from_f32<T>(s);
+}
+
+template <typename T, bool FAST>
+int launch_rows(const gbxm_window_attn_args& a, const Geo& g, int rc, int chunks, size_t lds, hipStream_t s) {
+  constexpr int PER = 16 / sizeof(T);
+  const bool vec = a.dk % PER == 0 && a.row_stride % PER == 0 && (a.H * a.dk) % PER == 0 &&
+                   (reinterpret_cast<uintptr_t>(a.qkv) | reinterpret_cast<uintptr_t>(a.kcache)) % 16 == 0;
+  // few rows: split every row's key tiles so that about two workgroups per CU exist (never more splits than tiles of a full window)
+  int splits = 1;
+  const int64_t groups = a.T * a.G * chunks;
+  if (a.partial && groups < 256) {
+    const int tiles = (a.window + KT - 1) / KT;
+    splits = static_cast<int>(std::min<int64_t>(std::min<int64_t>(512 / groups, tiles), a.partial_splits));
+    if (splits < 2) splits = 1;
+  }
+  const dim3 grid(a.T, a.G * chunks, splits);
+  const T* q = static_cast<const T*>(a.qkv);
+  const T* kc = static_cast<const T*>(a.kcache);
+  const T* vc = static_cast<const T*>(a.vcache);
+  T* out = static_cast<T*>(a.out);
+  float* part = static_cast<float*>(a.partial);
+  if (vec)
+    window_rows_kernel<T, FAST, true><<<grid, NT, lds, s>>>(q, a.row_stride, kc, vc, a.seq, a.tok, out, a.dist_mul, a.dist_rate, a.gate_bias, g, rc, splits, part);
+  else
+    window_rows_kernel<T, FAST, false><<<grid, NT, lds, s>>>(q, a.row_stride, kc, vc, a.seq, a.tok, out, a.dist_mul, a.dist_rate, a.gate_bias, g, rc, splits, part);
+  if (splits > 1) {
+    const int64_t n = a.T * a.H * a.dv;
+    window_reduce_kernel<T><<<dim3((n + NT - 1) / NT), NT, 0, s>>>(part, out, n, splits);
+  }
+  return after_launch("window_attention (rows)");
 }
 
 }  // namespace
@@ -124,22 +242,14 @@ extern "C" int gbxm_window_attention(const gbxm_window_attn_args* a, void* strea
   }
   Geo g{a->H, a->G, a->dk, a->dv, a->window, a->H * a->dk, a->G * a->dk, a->scale, a->softcap};
   const int R = a->H / a->G;
-  // query heads per workgroup: bounded by the value sums its threads can own and by 48 KB of LDS
-  int rc = R;
-  while (rc > 1 && (static_cast<int64_t>(rc) * a->dv > MAXACC * NT || static_cast<size_t>(rc) * (a->dk + KT) * 4 > 48 * 1024)) --rc;
-  if (static_cast<int64_t>(rc) * a->dv > MAXACC * NT || static_cast<size_t>(rc) * (a->dk + KT) * 4 > 48 * 1024)
-    return fail(GBXM_ERR_UNSUPPORTED, "window_attention: head sizes dk=%d dv=%d are beyond the row kernel", a->dk, a->dv);
+  // query heads per workgroup: at most RC, and the workgroup's LDS (rows, query, gates, the waves' sums) within 60 KB
+  if (a->dv > NCH * DCH) return fail(GBXM_ERR_UNSUPPORTED, "window_attention: value size %d beyond the row kernel (%d)", a->dv, NCH * DCH);
+  auto lds_of = [&](int rc_) { return static_cast<size_t>(2 * KT) * sizeof(void*) + static_cast<size_t>(rc_) * (a->dk + KT + 4 * a->dv) * sizeof(float); };
+  int rc = R < RC ? R : RC;
+  while (rc > 1 && lds_of(rc) > 60 * 1024) --rc;
+  if (lds_of(rc) > 60 * 1024) return fail(GBXM_ERR_UNSUPPORTED, "window_attention: head sizes dk=%d dv=%d are beyond the row kernel", a->dk, a->dv);
   const int chunks = (R + rc - 1) / rc;
-  const size_t lds = static_cast<size_t>(rc) * (a->dk + KT) * sizeof(float);
-  const dim3 grid(a->T, a->G * chunks);
-  if (a->T > 0x7fffffffLL || grid.y > 65535) return fail(GBXM_ERR_UNSUPPORTED, "window_attention: grid");
-  if (a->act == GBXM_BF16)
-    window_rows_kernel<bf16_t, true><<<grid, NT, lds, s>>>(static_cast<const bf16_t*>(a->qkv), a->row_stride, static_cast<const bf16_t*>(a->kcache),
-                                                           static_cast<const bf16_t*>(a->vcache), a->seq, a->tok, static_cast<bf16_t*>(a->out),
-                                                           a->dist_mul, a->dist_rate, a->gate_bias, g, rc);
-  else
-    window_rows_kernel<float, false><<<grid, NT, lds, s>>>(static_cast<const float*>(a->qkv), a->row_stride, static_cast<const float*>(a->kcache),
-                                                           static_cast<const float*>(a->vcache), a->seq, a->tok, static_cast<float*>(a->out),
-                                                           a->dist_mul, a->dist_rate, a->gate_bias, g, rc);
-  return after_launch("window_attention");
+  const size_t lds = lds_of(rc);
+  if (a->T > 0x7fffffffLL || a->G * chunks > 65535) return fail(GBXM_ERR_UNSUPPORTED, "window_attention: grid");
+  return a->act == GBXM_BF16 ? launch_rows<bf16_t, true>(*a, g, rc, chunks, lds, s) : launch_rows<float, false>(*a, g, rc, chunks, lds, s);
 }

@@ -34,37 +34,71 @@ __global__ __launch_bounds__(NT) void embed_kernel(const T* __restrict__ table, 
 template <typename T>
 __global__ __launch_bounds__(NT) void segment_rmsnorm_kernel(T* __restrict__ rows, int64_t stride, int n0, int n1, const float* __restrict__ w0,
                                                             const float* __restrict__ w1, float eps) {
+  constexpr int VR = 16;                   // values a thread keeps between the two passes
   __shared__ float red[NW];
   const int seg = blockIdx.y;
   T* p = rows + blockIdx.x * stride + (seg ? n0 : 0);
   const int n = seg ? n1 : n0;
   const float* w = seg ? w1 : w0;
+  float vr[VR];
   float ss = 0.f;
-  for (int c = threadIdx.x; c < n; c += NT) { const float v = to_f32(p[c]); ss += v * v; }
+#pragma unroll
+  for (int i = 0; i < VR; ++i) {
+    const int c = threadIdx.x + i * NT;
+    vr[i] = c < n ? to_f32(p[c]) : 0.f;
+    ss += vr[i] * vr[i];
+  }
+  for (int c = threadIdx.x + VR * NT; c < n; c += NT) { const float v = to_f32(p[c]); ss += v * v; }
   ss = block_sum<NW>(ss, red);
   const float r = 1.f / sqrtf(ss / n + eps);
-  for (int c = threadIdx.x; c < n; c += NT) p[c] = from_f32<T>(to_f32(p[c]) * r * w[c]);
+#pragma unroll
+  for (int i = 0; i < VR; ++i) {
+    const int c = threadIdx.x + i * NT;
+    if (c < n) p[c] = from_f32<T>(vr[i] * r * w[c]);
+  }
+  for (int c = threadIdx.x + VR * NT; c < n; c += NT) p[c] = from_f32<T>(to_f32(p[c]) * r * w[c]);
 }
+
+constexpr int ZR = 16;             // branch values a thread keeps between the statistic and the update (rows up to ZR * NT wide)
 
 template <typename T>
 __global__ __launch_bounds__(NT) void residual_norm_add_kernel(float* __restrict__ x, const T* __restrict__ branch, const float* __restrict__ mix,
                                                               const float* __restrict__ w, T* __restrict__ h, int width, int top, float eps,
                                                               float mult) {
   __shared__ float red[NW];
+  __shared__ float ml[64];
   const int64_t t = blockIdx.x;
   const T* b = branch + t * top * width;
-  const float* m = mix ? mix + t * top : nullptr;
+  const bool mixed = mix != nullptr;
+  if (mixed && threadIdx.x < min(top, 64)) ml[threadIdx.x] = mix[t * top + threadIdx.x];
+  __syncthreads();
   auto z_at = [&](int c) {
-    if (!m) return to_f32(b[c]);
+    if (!mixed) return to_f32(b[c]);
     float z = 0.f;
-    for (int s = 0; s < top; ++s) z += m[s] * to_f32(b[s * width + c]);
+    for (int s = 0; s < top; ++s) z += (s < 64 ? ml[s] : mix[t * top + s]) * to_f32(b[s * width + c]);
     return z;
   };
+  float zr[ZR];
   float ss = 0.f;
-  for (int c = threadIdx.x; c < width; c += NT) { const float z = z_at(c); ss += z * z; }
+#pragma unroll
+  for (int i = 0; i < ZR; ++i) {
+    const int c = threadIdx.x + i * NT;
+    zr[i] = c < width ? z_at(c) : 0.f;
+    ss += zr[i] * zr[i];
+  }
+  for (int c = threadIdx.x + ZR * NT; c < width; c += NT) { const float z = z_at(c); ss += z * z; }
   ss = block_sum<NW>(ss, red);
   const float r = 1.f / sqrtf(ss / width + eps);
-  for (int c = threadIdx.x; c < width; c += NT) {
+#pragma unroll
+  for (int i = 0; i < ZR; ++i) {
+    const int c = threadIdx.x + i * NT;
+    if (c < width) {
+      const float v = x[t * width + c] + mult * (zr[i] * r * w[c]);
+      x[t * width + c] = v;
+      if (h) h[t * width + c] = from_f32<T>(v);
+    }
+  }
+  for (int c = threadIdx.x + ZR * NT; c < width; c += NT) {
     const float v = x[t * width + c] + mult * (z_at(c) * r * w[c]);
     x[t * width + c] = v;
     if (h) h[t * width + c] = from_f32<T>(v);
@@ -83,24 +117,17 @@ __global__ __launch_bounds__(NT) void stream_rmsnorm_kernel(const float* __restr
   for (int c = threadIdx.x; c < width; c += NT) out[t * width + c] = from_f32<T>(x[t * width + c] * r * w[c]);
 }
 
-// One workgroup per row: wave v takes experts v, v + NW, ...; the logits meet in LDS, then `top` rounds of arg-max.
-template <typename T>
-__global__ __launch_bounds__(NT) void route_topk_kernel(const T* __restrict__ h, const float* __restrict__ router, int* __restrict__ idx,
-                                                       float* __restrict__ weight, int K, int E, int top, int renorm) {
+// Softmax over all experts and `top` rounds of arg-max on a row of fp32 router logits (the logits are a plain fp32 matrix product:
+// the vendor library's); one workgroup per row.
+__global__ __launch_bounds__(NT) void route_topk_kernel(const float* __restrict__ logits, int* __restrict__ idx, float* __restrict__ weight, int E,
+                                                       int top, int renorm) {
   extern __shared__ float lg[];            // [E] logits, then probabilities
   __shared__ float red[NW];
   __shared__ float bestv[NW];
   __shared__ int besti[NW];
   const int64_t t = blockIdx.x;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const T* hr = h + t * K;
-  for (int e = wave; e < E; e += NW) {
-    const float* wr = router + static_cast<int64_t>(e) * K;
-    float acc = 0.f;
-    for (int k = lane; k < K; k += 64) acc += wr[k] * to_f32(hr[k]);
-    acc = wave_sum(acc);
-    if (lane == 0) lg[e] = acc;
-  }
+  for (int e = threadIdx.x; e < E; e += NT) lg[e] = logits[t * E + e];
   __syncthreads();
   float mx = -INFINITY;
   for (int e = threadIdx.x; e < E; e += NT) mx = fmaxf(mx, lg[e]);
@@ -212,16 +239,13 @@ int gbxm_stream_rmsnorm(const float* x, const float* w, void* out, int64_t T_, i
   return after_launch("stream_rmsnorm");
 }
 
-int gbxm_route_topk(const void* h, const float* router, int32_t* idx, float* weight, int64_t T_, int32_t K, int32_t E, int32_t top,
-                    int32_t renorm, int32_t act, void* stream) {
-  if (!act_ok(act) || !h || !router || !idx || !weight || K <= 0 || E <= 0 || top < 1 || top > E || T_ < 0)
-    return fail(GBXM_ERR_INVALID, "route_topk: bad argument");
+int gbxm_route_topk(const float* logits, int32_t* idx, float* weight, int64_t T_, int32_t E, int32_t top, int32_t renorm, void* stream) {
+  if (!logits || !idx || !weight || E <= 0 || top < 1 || top > E || T_ < 0) return fail(GBXM_ERR_INVALID, "route_topk: bad argument");
   if (E > 8192) return fail(GBXM_ERR_UNSUPPORTED, "route_topk: more than 8192 experts");
   if (top > NT) return fail(GBXM_ERR_UNSUPPORTED, "route_topk: top > %d", NT);
   if (T_ == 0) return GBXM_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  GBXM_DISPATCH(act, (route_topk_kernel<T><<<dim3(T_), NT, E * sizeof(float), s>>>(static_cast<const T*>(h), router, idx, weight, K, E, top,
-                                                                                     renorm)));
+  route_topk_kernel<<<dim3(T_), NT, E * sizeof(float), s>>>(logits, idx, weight, E, top, renorm);
   return after_launch("route_topk");
 }
 

@@ -26,6 +26,7 @@ TABLE = {
     "GBX_GEMV_MX": ("0", "route the fused GEMV launches through libgbx_experimental.so's loader/consumer scaled-MFMA GEMV"),
     "GBX_PROMPT_GRAPH": ("1", "graph-replayed prompt buckets for 2..128-token prompts (0: eager pass)"),
     "GBX_DENSE_CACHE_GB": ("32", "budget of the resident dense weight images of long prompts, GiB (0 disables)"),
+    "GBX_STEP_GRAPH": ("1", "BatchScheduler: decode-only steps of a recurring set of slots replayed from a HIP graph (0: eager launches) (A/B)"),
     "GBX_TP_GRAPH": ("1", "bench.py: RCCL collectives inside the HIP graph (0: eager launches)"),
     "GBX_TP_P2P": ("0", "bench.py: one-shot P2P all-reduce instead of RCCL (falls back to RCCL, with the reason reported, where it cannot work)"),
 }

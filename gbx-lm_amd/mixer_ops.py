@@ -84,14 +84,15 @@ def stream_rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float, act_dtype: torc
 
 
 def route_topk(h: torch.Tensor, router: torch.Tensor, top: int, renormalize: bool = False):
-    act = _act(h, "h")
-    h = h.contiguous()
-    t, k = h.shape
-    e = router.shape[0]
+    """(idx int32 [T, top], weights fp32 [T, top]).  The logits are an fp32 product of the rows (their bf16 image widened, when
+    activations are bf16) with the fp32 router -- the vendor library's GEMM / GEMV; softmax and the choice are one launch."""
+    _act(h, "h")
+    logits = torch.matmul(h if h.dtype == torch.float32 else h.float(), _f32(router, "router").t())
+    t, e = logits.shape
     idx = torch.empty((t, top), dtype=torch.int32, device=h.device)
     w = torch.empty((t, top), dtype=torch.float32, device=h.device)
-    _lib.check_mixers(_lib.mixers().gbxm_route_topk(h.data_ptr(), _f32(router, "router").data_ptr(), idx.data_ptr(), w.data_ptr(), t, k, e, top,
-                                                   int(bool(renormalize)), act, _stream(h.device)))
+    _lib.check_mixers(_lib.mixers().gbxm_route_topk(logits.data_ptr(), idx.data_ptr(), w.data_ptr(), t, e, top, int(bool(renormalize)),
+                                                   _stream(h.device)))
     return idx, w
 
 
@@ -125,12 +126,16 @@ def window_attention(qkv: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tens
     if tuple(kcache.shape[1:]) != (m.window, m.nk) or tuple(vcache.shape[1:]) != (m.window, m.nv) or kcache.shape[0] <= max(batch.slot):
         raise ValueError("window_attention: caches do not fit the module or the step's slots")
     out = torch.empty((batch.total, m.heads * m.vdim), dtype=qkv.dtype, device=qkv.device)
+    partial, splits = None, 0
+    if batch.total * m.kv_heads < 256 and m.window > 128:     # few rows, long windows: room for key-split partial sums
+        splits = min(16, (m.window + 63) // 64)
+        partial = torch.empty((splits, batch.total, m.heads * m.vdim), dtype=torch.float32, device=qkv.device)
     a = _lib.WindowAttnArgs(qkv.data_ptr(), qkv.stride(0), kcache.data_ptr(), vcache.data_ptr(), batch.seq.data_ptr(), batch.tok.data_ptr(),
                             batch.tiles.data_ptr() if batch.tiles is not None and batch.tiles.numel() else None, out.data_ptr(),
                             _f32(m.dist_mul, "dist_mul").data_ptr(), _f32(m.dist_rate, "dist_rate").data_ptr(),
                             _f32(m.gate_bias, "gate_bias").data_ptr(), batch.total, len(batch.slot),
                             0 if batch.tiles is None else batch.tiles.shape[0], batch.q_tile, m.heads, m.kv_heads, m.dim, m.vdim, m.window,
-                            m.scale, m.softcap, int(batch.decode_only), act)
+                            m.scale, m.softcap, int(batch.decode_only), act, None if partial is None else partial.data_ptr(), splits)
     _lib.check_mixers(_lib.mixers().gbxm_window_attention(ctypes.byref(a), _stream(qkv.device)))
     return out
 

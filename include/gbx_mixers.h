@@ -33,13 +33,14 @@ int gbxm_residual_norm_add(float* x, const void* branch, const float* mix, const
                            int32_t top, float eps, float mult, int32_t act, void* stream);
 /* out[t] = rms_norm(x[t]) * w in the activation dtype. */
 int gbxm_stream_rmsnorm(const float* x, const float* w, void* out, int64_t T, int32_t width, float eps, int32_t act, void* stream);
-/* Router: logits = router (fp32 [E][K]) . h[t], probabilities over all E, the `top` largest (ties: lower index); weights are
- * the probabilities, divided by their sum if renorm. */
-int gbxm_route_topk(const void* h, const float* router, int32_t* idx, float* weight, int64_t T, int32_t K, int32_t E, int32_t top,
-                    int32_t renorm, int32_t act, void* stream);
+/* Router decisions from fp32 logits [T][E] (a plain matrix product, left to the vendor library): probabilities over all E, the
+ * `top` largest (ties: lower index); weights are the probabilities, divided by their sum if renorm. */
+int gbxm_route_topk(const float* logits, int32_t* idx, float* weight, int64_t T, int32_t E, int32_t top, int32_t renorm, void* stream);
 /* y[t][s] = down[e] (silu(gate[e] h[t]) * (up[e] h[t])), e = idx[t][s]; gate_up [E][2F][K] (gate rows, then up rows),
- * down [E][K][F].  `ws` (bytes from gbxm_expert_glu_workspace) lets prompt-sized steps run as grouped matrix-core products. */
+ * down [E][K][F].  `ws`: gbxm_expert_glu_workspace bytes (hidden rows; for prompt-sized bf16 steps also the expert-sorted order of
+ * the grouped matrix-core products -- gbxm_expert_glu_grouped tells which of the two a call takes). */
 size_t gbxm_expert_glu_workspace(int64_t T, int32_t K, int32_t F, int32_t E, int32_t top, int32_t act);
+int gbxm_expert_glu_grouped(int64_t T, int32_t K, int32_t F, int32_t E, int32_t top, int32_t act);
 int gbxm_expert_glu(const void* h, const void* gate_up, const void* down, const int32_t* idx, void* y, int64_t T, int32_t K,
                     int32_t F, int32_t E, int32_t top, int32_t act, void* ws, size_t ws_bytes, void* stream);
 
@@ -63,6 +64,8 @@ typedef struct {
   float scale, softcap;
   int32_t decode_only;          /* every sequence brings one row */
   int32_t act;
+  void* partial;                /* optional fp32 [partial_splits][T][H*dv]: lets a step of few rows split its keys over workgroups */
+  int32_t partial_splits;
 } gbxm_window_attn_args;
 int gbxm_window_attention(const gbxm_window_attn_args* a, void* stream);
 /* 1 if a step of this kind runs on the matrix-core tile kernel, 0 if on the row kernel (tests and benchmarks name the kernel). */

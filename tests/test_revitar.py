@@ -310,7 +310,7 @@ def test_expert_mechanism(device, dtype, rows, k, f, experts, top):
     idx[: rows // 2, 0] = 0 if top == 1 else idx[: rows // 2, 0]
     if device == "cuda":
         from gbx_lm_amd import mixer_ops as M, _lib
-        grouped = _lib.mixers().gbxm_expert_glu_workspace(rows, k, f, experts, top, _lib.GBXM_BF16 if dtype == torch.bfloat16 else _lib.GBXM_F32) > 0
+        grouped = _lib.mixers().gbxm_expert_glu_grouped(rows, k, f, experts, top, _lib.GBXM_BF16 if dtype == torch.bfloat16 else _lib.GBXM_F32) == 1
         assert grouped == (dtype == torch.bfloat16 and rows * top >= 256 and k % 32 == 0 and f % 32 == 0)
         y = M.expert_glu(h.to(device), m.gate_up, m.down, idx.to(device))
     else:
