@@ -378,3 +378,25 @@ def test_loader_reads_every_size_from_the_config(checkpoints, tmp_path):
     odd = O.make_config([{"type": "convolution", "mixer": {}, "mlp": None}])
     with pytest.raises(ValueError):
         load_model(O.save_checkpoint(str(tmp_path / "odd"), odd, {"embed": torch.zeros(1)}), device="cpu")
+
+
+def test_command_line_and_samplers(checkpoints, capsys):
+    """``python -m gbx_lm_amd.cli``: one prompt through generate_step, several through the scheduler; greedy output equals the
+    loops' own; the temperature / top-p sampler is reproducible from its seed and never leaves the nucleus."""
+    import json
+    from gbx_lm_amd import cli as G
+    path, cfg, w = checkpoints["mixed"]
+    p1, p2 = tokens_for(cfg, 6, 70), tokens_for(cfg, 13, 71)
+    ids = lambda p: ",".join(map(str, p))
+    assert G.main(["--model", path, "--prompt-ids", ids(p1), "--max-tokens", "5", "--dtype", "float32"]) == 0
+    one = json.loads(capsys.readouterr().out.strip().splitlines()[-1])
+    assert G.main(["--model", path, "--prompt-ids", ids(p1), "--prompt-ids", ids(p2), "--max-tokens", "5", "--dtype", "float32"]) == 0
+    two = [json.loads(l) for l in capsys.readouterr().out.strip().splitlines()[-2:]]
+    assert one["tokens"] == two[0]["tokens"] and len(two[1]["tokens"]) == 5 and two[1]["prompt_tokens"] == 13
+    lp = torch.log_softmax(torch.tensor([[4.0, 3.0, 0.0, -1.0, -9.0]]), -1).repeat(200, 1)
+    s1, s2 = G.make_sampler(0.8, 0.9, seed=4)(lp), G.make_sampler(0.8, 0.9, seed=4)(lp)
+    assert torch.equal(s1, s2) and set(s1.tolist()) <= {0, 1} and len(set(s1.tolist())) == 2
+    assert G.make_sampler(0.0) is None
+    model = model_for(checkpoints, "mixed", "cpu", torch.float32)
+    sampled = BatchScheduler(model).generate([p1, p2], max_tokens=4, sampler=G.make_sampler(1.0, 0.95, seed=1))
+    assert [len(o) for o in sampled] == [4, 4] and all(0 <= t < cfg["vocab"] for o in sampled for t in o)
