@@ -558,7 +558,7 @@ def revitar_bench(args):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--design", default=None, choices=["revitar"], help="side benchmark of one model design beside the closest existing "
-                    "family at equal size (own JSON line; the default workload and its contract are unchanged)")
+                    "family at equal size (own JSON line; the default workload and its output are unchanged)")
     ap.add_argument("--sizes", default="small,a3b-like", help="--design revitar: comma-separated names of REVITAR_SIZES")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=512, help="timed decode steps (default: > 0.5 s of GPU time, so that a coarse GPU-busy sampler sees the run)")

@@ -23,12 +23,13 @@ MIXED = O.make_config([
     O.attention_layer(4, 2, 32, 32, window=5, mlp=O.moe(5, 2, 32)),
     O.attention_layer(2, 2, 16, 48, window=300, softcap=None, mlp=None),                 # one kv head per head, window > sequence
     O.attention_layer(4, 1, 64, 64, window=17, scale=0.21, softcap=3.0, mlp=O.moe(3, 1, 48)),
-    O.attention_layer(3, 1, 24, 8, window=1, mlp=O.moe(4, 4, 16)),                        # sees itself only; every expert chosen
+    O.attention_layer(3, 1, 20, 7, window=1, mlp=O.moe(4, 4, 16)),                        # sees itself only; every expert chosen; odd sizes
 ], vocab=61, width=64, residual_mult=0.5, embed_scale=2.0)
 PLAIN = O.make_config([
     O.attention_layer(2, 1, 64, 128, window=130, mlp=O.moe(8, 2, 64)),                    # a window that ends inside a second query tile
     O.attention_layer(8, 2, 32, 32, window=33, mlp=None),
-], vocab=40, width=128, eps=1e-6, residual_mult=1.0, embed_scale=1.0)
+    O.attention_layer(6, 3, 12, 10, window=9, mlp=O.moe(3, 2, 20)),                       # nothing a multiple of 8
+], vocab=40, width=136, eps=1e-6, residual_mult=1.0, embed_scale=1.0)
 
 
 @pytest.fixture(scope="module")
@@ -185,6 +186,18 @@ def test_slots_are_reused(checkpoints, device):
     assert O.rel_err(torch.cat(got_c), O.forward(c, cfg, w)) < TOL[torch.float32]
     assert O.rel_err(torch.cat(got_b), O.forward(b[:46], cfg, w)[40:46]) < TOL[torch.float32]
     eng.release("b"); eng.release("c")
+    # more sequences than slots exist: the rings grow (and keep what they hold) while "d" is in the middle of its sequence
+    d = tokens_for(cfg, 30, 23)
+    others = [tokens_for(cfg, 5 + i, 24 + i) for i in range(4)]
+    got_d = [eng.step([("d", d[:12])], [all_places(12)])]
+    before = eng.caches[0].keys.shape[0]
+    out = eng.step([("d", d[12:20])] + [(("o", i), o) for i, o in enumerate(others)], [all_places(8)] + [[len(o) - 1] for o in others])
+    assert eng.caches[0].keys.shape[0] > before
+    got_d.append(out[:8])
+    got_d.append(eng.step([("d", d[20:])], [all_places(10)]))
+    assert O.rel_err(torch.cat(got_d), O.forward(d, cfg, w)) < TOL[torch.float32]
+    for i, o in enumerate(others):
+        assert O.rel_err(out[8 + i][None], O.forward(o, cfg, w)[-1:]) < TOL[torch.float32]
     with pytest.raises(KeyError):
         eng.release("c")
     tight = BatchScheduler(model, max_tokens=10)
@@ -370,6 +383,7 @@ def test_loader_reads_every_size_from_the_config(checkpoints, tmp_path):
     assert (at.heads, at.kv_heads, at.dim, at.vdim, at.window, at.softcap) == (4, 1, 64, 64, 17, 3.0) and abs(at.scale - 0.21) < 1e-12
     assert model.layers[1].mlp is None and model.layers[1].norm2 is None and model.layers[1].mixer.softcap == 0.0
     assert model.layers[3].mlp.top == 4 and model.layers[0].mlp.router.dtype == torch.float32
+    assert (model.layers[3].mixer.dim, model.layers[3].mixer.vdim, model.layers[3].mixer.window) == (20, 7, 1)
     assert model.model.embed_tokens.weight.dtype == torch.bfloat16 and model.layers[0].norm1.weight.dtype == torch.float32
     broken = dict(w)
     del broken["l2.mix.pb"]
