@@ -1,7 +1,7 @@
 // Matrix-core kernel of gated sliding-window attention for bf16 prompt portions (mechanism: mixers_attn.hip).
 //
 // One workgroup = 4 waves = one tile of up to 128 query rows of one (sequence, head); a wave owns 32 queries.  Key / value tiles
-// of 32 positions go global -> LDS once per workgroup (ring rows for positions before the step, projection rows inside it; rows
+// of 32 positions go global -> registers (one tile ahead) -> LDS once per workgroup (ring rows for positions before the step, projection rows inside it; rows
 // past the tile's last query are zero-filled so that a zero gate never meets a stale NaN).  Both products are computed swapped so
 // that a lane owns ONE query and the gate arithmetic is lane-local:
 //   S^T[key, q] = mfma(K rows, Q rows)      lane (q = lane % 32) holds 16 keys of the tile, the other 16 are in lane ^ 32
@@ -74,21 +74,38 @@ __global__ __launch_bounds__(256) void window_tile_kernel(const TileArgs a) {
     return j < pos0 ? ring + (static_cast<int64_t>(slot) * W + j % W) * row_elems : a.qkv + (row0 + (j - pos0)) * a.stride + seg_off;
   };
 
+  // key / value tile: global -> registers one tile ahead, registers -> LDS at the top of its iteration
+  constexpr int KP = (KT * (DK / 8) + 255) / 256, VP = (KT * (DV / 8) + 255) / 256;
+  u32x4 kr[KP], vr[VP];
+  auto fetch = [&](int jt) {
+#pragma unroll
+    for (int i = 0; i < KP; ++i) {
+      const int p = tid + 256 * i, row = p / (DK / 8), c = p % (DK / 8), j = jt + row;
+      kr[i] = u32x4{0, 0, 0, 0};
+      if (p < KT * (DK / 8) && j <= jlast) kr[i] = *reinterpret_cast<const u32x4*>(src(a.kc, nkv_k, a.nq, j) + kvh * DK + c * 8);
+    }
+#pragma unroll
+    for (int i = 0; i < VP; ++i) {
+      const int p = tid + 256 * i, row = p / (DV / 8), c = p % (DV / 8), j = jt + row;
+      vr[i] = u32x4{0, 0, 0, 0};
+      if (p < KT * (DV / 8) && j <= jlast) vr[i] = *reinterpret_cast<const u32x4*>(src(a.vc, nkv_v, a.nq + a.nk, j) + kvh * DV + c * 8);
+    }
+  };
+  fetch(jfirst);
   for (int jt = jfirst; jt <= jlast; jt += KT) {
     __syncthreads();                                          // the previous tile has been consumed
-    for (int p = tid; p < KT * (DK / 8); p += 256) {
-      const int row = p / (DK / 8), c = p % (DK / 8), j = jt + row;
-      u32x4 v = u32x4{0, 0, 0, 0};
-      if (j <= jlast) v = *reinterpret_cast<const u32x4*>(src(a.kc, nkv_k, a.nq, j) + kvh * DK + c * 8);
-      *reinterpret_cast<u32x4*>(kl + row * KROW + c * 16) = v;
+#pragma unroll
+    for (int i = 0; i < KP; ++i) {
+      const int p = tid + 256 * i;
+      if (p < KT * (DK / 8)) *reinterpret_cast<u32x4*>(kl + (p / (DK / 8)) * KROW + (p % (DK / 8)) * 16) = kr[i];
     }
-    for (int p = tid; p < KT * (DV / 8); p += 256) {
-      const int row = p / (DV / 8), c = p % (DV / 8), j = jt + row;
-      u32x4 v = u32x4{0, 0, 0, 0};
-      if (j <= jlast) v = *reinterpret_cast<const u32x4*>(src(a.vc, nkv_v, a.nq + a.nk, j) + kvh * DV + c * 8);
-      *reinterpret_cast<u32x4*>(vl + row * VROW + c * 16) = v;
+#pragma unroll
+    for (int i = 0; i < VP; ++i) {
+      const int p = tid + 256 * i;
+      if (p < KT * (DV / 8)) *reinterpret_cast<u32x4*>(vl + (p / (DV / 8)) * VROW + (p % (DV / 8)) * 16) = vr[i];
     }
     __syncthreads();
+    if (jt + KT <= jlast) fetch(jt + KT);                     // the next tile travels while this one is computed
     if (!wave_live || jt > wq1 || jt + KT - 1 < wq0 - W + 1) continue;      // wave-uniform: no key of the tile is seen by this wave
 
     f32x16 st = f32x16{0};
