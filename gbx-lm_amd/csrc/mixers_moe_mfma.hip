@@ -101,19 +101,19 @@ __global__ __launch_bounds__(256) void expert_up_kernel(const bf16_t* __restrict
 
   auto chunk = [&](int k0, auto steps_c) {
     constexpr int S = decltype(steps_c)::value;                         // MFMA steps of the chunk: 4 (64 elements) or 2 (32)
+    const int off = k0 + hb * (S * 8);
+    u32x4 fg[S], fu[S];                                                 // weight fragments: requested ahead of the tile hand-over
+#pragma unroll
+    for (int i = 0; i < S; ++i) {
+      fg[i] = *reinterpret_cast<const u32x4*>(wgl + off + i * 8);
+      fu[i] = *reinterpret_cast<const u32x4*>(wul + off + i * 8);
+    }
     __syncthreads();                                                    // the previous chunk's fragments have been read
     b.park(bl);
     __syncthreads();
     const int kn = k0 + S * 16;
     if (kn < K) b.fetch(kn, kn + 64 <= K ? 8 : 4);                      // the next chunk travels while this one is multiplied
     if (!live) return;
-    const int off = k0 + hb * (S * 8);
-    u32x4 fg[S], fu[S];
-#pragma unroll
-    for (int i = 0; i < S; ++i) {
-      fg[i] = *reinterpret_cast<const u32x4*>(wgl + off + i * 8);
-      fu[i] = *reinterpret_cast<const u32x4*>(wul + off + i * 8);
-    }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       u32x4 fb[S];
@@ -177,12 +177,6 @@ __global__ __launch_bounds__(256) void expert_down_kernel(const bf16_t* __restri
 
   auto chunk = [&](int f0_, auto steps_c) {
     constexpr int S = decltype(steps_c)::value;
-    __syncthreads();
-    b.park(bl);
-    __syncthreads();
-    const int fn = f0_ + S * 16;
-    if (fn < F) b.fetch(fn, fn + 64 <= F ? 8 : 4);
-    if (!live) return;
     const int off = f0_ + hb * (S * 8);
     u32x4 fa[2][S];
 #pragma unroll
@@ -190,6 +184,12 @@ __global__ __launch_bounds__(256) void expert_down_kernel(const bf16_t* __restri
       fa[0][i] = *reinterpret_cast<const u32x4*>(wl[0] + off + i * 8);
       fa[1][i] = *reinterpret_cast<const u32x4*>(wl[1] + off + i * 8);
     }
+    __syncthreads();
+    b.park(bl);
+    __syncthreads();
+    const int fn = f0_ + S * 16;
+    if (fn < F) b.fetch(fn, fn + 64 <= F ? 8 : 4);
+    if (!live) return;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       u32x4 fb[S];
