@@ -178,9 +178,14 @@ template <typename T>
 __global__ __launch_bounds__(NT) void window_reduce_kernel(const float* __restrict__ partial, T* __restrict__ out, int64_t n, int splits) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * NT + threadIdx.x;
   if (i >= n) return;
-  float s = 0.f;
-  for (int z = 0; z < splits; ++z) s += partial[z * n + i];
-  out[i] = from_f32<T>(s);
+  float s4[4] = {0.f, 0.f, 0.f, 0.f};                 // four running sums (split z goes to sum z % 4): the loads of a row do not wait
+  int z = 0;                                          // for each other; the order is fixed all the same
+  for (; z + 4 <= splits; z += 4) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) s4[u] += partial[(z + u) * n + i];
+  }
+  for (; z < splits; ++z) s4[z & 3] += partial[z * n + i];
+  out[i] = from_f32<T>((s4[0] + s4[1]) + (s4[2] + s4[3]));
 }
 
 template <typename T, bool FAST>

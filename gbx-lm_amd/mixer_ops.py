@@ -128,8 +128,10 @@ def window_attention(qkv: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tens
     out = torch.empty((batch.total, m.heads * m.vdim), dtype=qkv.dtype, device=qkv.device)
     partial, splits = None, 0
     if batch.total * m.kv_heads < 256 and m.window > 128:     # few rows, long windows: room for key-split partial sums
-        splits = min(64, (m.window + 63) // 64)
-        partial = torch.empty((splits, batch.total, m.heads * m.vdim), dtype=torch.float32, device=qkv.device)
+        keys = max(min(m.window, p + n) for p, n in zip(batch.pos0, batch.n_new))      # the longest key range a row of this step has
+        splits = min(64, (keys + 63) // 64)
+        if splits > 1:
+            partial = torch.empty((splits, batch.total, m.heads * m.vdim), dtype=torch.float32, device=qkv.device)
     a = _lib.WindowAttnArgs(qkv.data_ptr(), qkv.stride(0), kcache.data_ptr(), vcache.data_ptr(), batch.seq.data_ptr(), batch.tok.data_ptr(),
                             batch.tiles.data_ptr() if batch.tiles is not None and batch.tiles.numel() else None, out.data_ptr(),
                             _f32(m.dist_mul, "dist_mul").data_ptr(), _f32(m.dist_rate, "dist_rate").data_ptr(),
