@@ -248,7 +248,7 @@ def write_checkpoint(path: str, config: Dict, strategy: Optional[Dict], seed: in
 
 # ------------------------------------------------------------------------------------------------ Revitar (dense, ragged steps)
 def revitar_config(width: int, heads: int, kv_heads: int, dim: int, vdim: int, window: int, experts: int, top: int, ff: int,
-                   n_layers: int, vocab: int = 32000, softcap: float = 50.0, residual_mult: float = 0.3, embed_scale: float = 1.0) -> Dict:
+                   n_layers: int, vocab: int = 32000, softcap: float = 30.0, residual_mult: float = 0.5, embed_scale: float = 1.0) -> Dict:
     """config.json of a Revitar model whose layers are all alike (benchmarks; a checkpoint may mix layers freely)."""
     layer = {"type": "attention",
              "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "mask": {"size": window},

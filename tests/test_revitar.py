@@ -414,3 +414,65 @@ def test_command_line_and_samplers(checkpoints, capsys):
     model = model_for(checkpoints, "mixed", "cpu", torch.float32)
     sampled = BatchScheduler(model).generate([p1, p2], max_tokens=4, sampler=G.make_sampler(1.0, 0.95, seed=1))
     assert [len(o) for o in sampled] == [4, 4] and all(0 <= t < cfg["vocab"] for o in sampled for t in o)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("width", [24, 136, 4500])
+def test_norm_residual_and_embedding_mechanisms(device, dtype, width):
+    """The stream update x += m * N(branch) * w alone (plain branch, and top candidate rows mixed by fp32 weights), the last norm,
+    the whole-segment norms of q | k rows and the scaled embedding; rows wider than one pass of a workgroup included."""
+    from gbx_lm_amd.models.residual import BranchNormResidual, StreamRMSNorm
+    g = torch.Generator().manual_seed(width)
+    rows, top, eps, mult = 5, 3, 1e-5, 0.7
+    tol = 1e-5 if dtype == torch.float32 else 1e-2
+    x0 = torch.randn((rows, width), generator=g)
+    w = torch.rand((width,), generator=g) + 0.5
+    for mix in (None, torch.rand((rows, top), generator=g)):
+        branch = torch.randn((rows, width) if mix is None else (rows, top, width), generator=g).to(dtype)
+        m = BranchNormResidual(width, eps, mult)
+        m.weight.copy_(w)
+        m.to(device)
+        x = x0.clone().to(device)
+        h = m(x, branch.to(device), None if mix is None else mix.to(device), dtype)
+        z = branch.to(O.F64) if mix is None else (branch.to(O.F64) * mix.to(O.F64)[..., None]).sum(1)
+        ref = x0.to(O.F64) + mult * O.rms(z, w.to(O.F64), eps)
+        assert O.rel_err(x, ref) < 1e-5 and h.dtype == dtype and O.rel_err(h, ref) < tol
+    n = StreamRMSNorm(width, eps)
+    n.weight.copy_(w)
+    n.to(device)
+    assert O.rel_err(n(x0.to(device), dtype), O.rms(x0.to(O.F64), w.to(O.F64), eps)) < tol
+    # segment norms: q (2/3 of the row) and k (1/6) normalised each over its whole segment, v untouched
+    if device == "cuda":
+        from gbx_lm_amd import mixer_ops as M
+        n0, n1 = 4 * (width // 6), width // 6
+        qkv = torch.randn((rows, width), generator=g).to(dtype)
+        w0, w1 = torch.rand((n0,), generator=g) + 0.5, torch.rand((n1,), generator=g) + 0.5
+        out = qkv.clone().to(device)
+        M.segment_rmsnorm_(out, n0, n1, w0.to(device), w1.to(device), eps)
+        assert O.rel_err(out[:, :n0], O.rms(qkv[:, :n0].to(O.F64), w0.to(O.F64), eps)) < tol
+        assert O.rel_err(out[:, n0:n0 + n1], O.rms(qkv[:, n0:n0 + n1].to(O.F64), w1.to(O.F64), eps)) < tol
+        assert torch.equal(out[:, n0 + n1:].cpu(), qkv[:, n0 + n1:])
+        table = torch.randn((11, width), generator=g).to(dtype)
+        toks = torch.tensor([3, 0, 10, 3])
+        xe, he = M.embed_scaled(table.to(device), toks.to(device), 0.37)
+        assert O.rel_err(xe, table[toks].to(O.F64) * 0.37) < 1e-6 and he.dtype == dtype
+
+
+@pytest.mark.gpu
+def test_decode_steps_are_replayed_from_a_graph(checkpoints):
+    """From its third occurrence a decode-only step of the same slots runs as one HIP-graph replay; replays (with eager prompt steps
+    of other sequences between them, and the rings re-allocated once) must keep agreeing with the oracle."""
+    _, cfg, w = checkpoints["mixed"]
+    model = model_for(checkpoints, "mixed", "cuda", torch.float32)
+    a, b = tokens_for(cfg, 40, 90), tokens_for(cfg, 12, 91)
+    eng = BatchScheduler(model)
+    got = [eng.step([("a", a[:10])], [all_places(10)])]
+    for i in range(10, 25):
+        got.append(eng.step([("a", [a[i]])]))
+    assert eng._graphs and all(gr.graph is not None for gr in eng._graphs.values())
+    other = eng.step([("b", b)], [all_places(len(b))])                    # a second slot: the rings grow, captured pointers are stale
+    for i in range(25, 40):
+        got.append(eng.step([("a", [a[i]])]))
+    assert O.rel_err(torch.cat(got), O.forward(a, cfg, w)) < TOL[torch.float32]
+    assert O.rel_err(other, O.forward(b, cfg, w)) < TOL[torch.float32]
