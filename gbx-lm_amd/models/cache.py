@@ -166,3 +166,88 @@ class WindowKVCache:
 
     def is_trimmable(self):
         return False
+
+
+class SlotKVCache:
+    """Rows of a softmax-attention mixer for several sequences, token-major ``[slots, rows, width]``.  Position ``p`` of a sequence
+    lives in row ``p`` while ``p < keep`` (the first tokens of a sequence, which a window mask may keep visible for ever) and in row
+    ``keep + (p - keep) % ring`` afterwards.  Two shapes of the same table:
+
+    * a window: ``ring = window`` rows are enough for every key a later query can still see;
+    * no window (``window=None``): ``keep = 0`` and the ring is the whole capacity, which doubles when a sequence outgrows it
+      (row = position while it fits, so a larger table is the old one copied in front).
+
+    ``v_width = 0`` stores one row per token only (a mixer whose values are a part of its key rows: ``values`` is ``keys``).  As
+    with ``WindowKVCache`` a step's own tokens are read from the step and appended after it has attended."""
+
+    def __init__(self, k_width: int, v_width: int, window: Optional[int], keep: int = 0, slots: Optional[SequenceSlots] = None,
+                 first_capacity: int = 256):
+        self.k_width, self.v_width = int(k_width), int(v_width)
+        self.window = None if window is None else int(window)
+        self.keep = 0 if window is None else min(int(keep), 1 << 30)
+        self.ring = first_capacity if window is None else self.window
+        self.slots = slots if slots is not None else SequenceSlots(1)
+        self.slots.listeners.append(self)
+        self.keys = None
+        self.values = None
+
+    @property
+    def offset(self) -> int:
+        return max(self.slots.length[0], 0)
+
+    @property
+    def rows(self) -> int:
+        return self.keep + self.ring
+
+    def row_of(self, pos: torch.Tensor) -> torch.Tensor:
+        return torch.where(pos < self.keep, pos, self.keep + (pos - self.keep) % self.ring)
+
+    def _alloc(self, n_slots: int, dtype, device) -> None:
+        self.keys = torch.zeros((n_slots, self.rows, self.k_width), dtype=dtype, device=device)
+        self.values = torch.zeros((n_slots, self.rows, self.v_width), dtype=dtype, device=device) if self.v_width else self.keys
+
+    def reserve(self, longest: int, dtype, device) -> None:
+        """Room for sequences of up to ``longest`` tokens (allocates at first use; a windowed table never grows in rows)."""
+        if self.window is None and longest > self.ring:
+            old_k, old_v, old_rows = self.keys, self.values, self.ring
+            while self.ring < longest:
+                self.ring *= 2
+            if old_k is not None:
+                self._alloc(old_k.shape[0], old_k.dtype, old_k.device)
+                self.keys[:, :old_rows] = old_k
+                if self.v_width:
+                    self.values[:, :old_rows] = old_v
+        if self.keys is None:
+            self._alloc(self.slots.n_slots, dtype, device)
+
+    def ensure(self, longest: int) -> None:
+        """Growth check for callers that replay captured launches (no allocation may happen inside a replay)."""
+        if self.keys is not None:
+            self.reserve(longest, self.keys.dtype, self.keys.device)
+
+    def grow(self, n_slots: int) -> None:
+        if self.keys is not None and self.keys.shape[0] < n_slots:
+            old_k, old_v = self.keys, self.values
+            self._alloc(max(n_slots, 2 * old_k.shape[0]), old_k.dtype, old_k.device)
+            self.keys[:old_k.shape[0]] = old_k
+            if self.v_width:
+                self.values[:old_v.shape[0]] = old_v
+
+    def stored(self, pos0: int) -> torch.Tensor:
+        """Positions before ``pos0`` whose rows are still in the table, ascending."""
+        first = max(self.keep, pos0 - self.ring)
+        return torch.cat([torch.arange(0, min(self.keep, pos0)), torch.arange(first, max(first, pos0))])
+
+    def append_rows(self, k: torch.Tensor, v: Optional[torch.Tensor], slot: int, pos0: int) -> None:
+        """Plain-torch append of one sequence's new rows in order (the HIP path appends a whole step in one launch)."""
+        n = k.shape[0]
+        rows = self.row_of(torch.arange(pos0, pos0 + n))
+        last = {int(r): i for i, r in enumerate(rows.tolist())}                  # a later row of the step takes the same place
+        idx = torch.tensor(sorted(last.values()), dtype=torch.long)
+        at = rows[idx].to(k.device)
+        self.keys[slot, at] = k[idx.to(k.device)]
+        if self.v_width:
+            self.values[slot, at] = v[idx.to(k.device)]
+
+    def is_trimmable(self):
+        return False

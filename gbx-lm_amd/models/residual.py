@@ -43,3 +43,13 @@ class StreamRMSNorm(nn.Module):
             from .. import mixer_ops as M
             return M.stream_rmsnorm(x, self.weight, self.eps, act_dtype)
         return (x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + self.eps) * self.weight.float()).to(act_dtype)
+
+
+def stream_add_(x: torch.Tensor, a: torch.Tensor, b: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x += a (+ b) in fp32 on the fp32 stream: the update of a layer whose sublayers all read one norm of the stream and whose
+    outputs (activation dtype) are added together.  GPU tensors: one launch."""
+    if x.is_cuda:
+        from .. import mixer_ops as M
+        return M.stream_add_(x, a, b)
+    y = a.float() if b is None else a.float() + b.float()
+    return x.add_(y)

@@ -21,8 +21,8 @@ from torch import nn
 
 from ..batching import StepBatch
 from .base import BaseModelArgs
-from .cache import SequenceSlots
 from .residual import BranchNormResidual, StreamRMSNorm
+from .step_model import RaggedStepModel
 from .switch_layers import DenseRoutedGLU
 from .window_attention import GatedWindowAttention
 
@@ -95,32 +95,10 @@ class RevitarModel(nn.Module):
         return x, (x if w.dtype == torch.float32 else x.to(w.dtype))
 
 
-class Model(nn.Module):
-    quantized = False                       # dense checkpoint: the loader skips the GBA strategy / re-initialisation
-
+class Model(RaggedStepModel):
     def __init__(self, args: ModelArgs):
-        super().__init__()
-        self.args = args
-        self.model_type = args.model_type
+        super().__init__(args)
         self.model = RevitarModel(args)
-        self.lm_head = nn.Linear(args.width, args.vocab, bias=False)
-        self.lm_head.weight.requires_grad_(False)
-        self.trace_layers = None            # a list collects the fp32 stream after every layer (diagnostics, tests)
-
-    @property
-    def layers(self):
-        return self.model.layers
-
-    def required_kernels(self) -> None:
-        """Load (and, in a checkout without built files, first compile) the one kernel library this model runs on."""
-        from .. import _lib
-        _lib.mixers()
-
-    def make_cache(self) -> List[Any]:
-        """Per-layer caches over one shared slot table; slot 0 is handed to the one-sequence generate loop."""
-        slots = SequenceSlots(1)
-        slots.length[0] = 0
-        return [layer.mixer.make_cache(slots) for layer in self.model.layers]
 
     def forward_tokens(self, tokens: torch.Tensor, batch: StepBatch, caches) -> torch.Tensor:
         """One ragged step: tokens [T] -> fp32 stream [T, width] after the last layer.  Positions are NOT advanced here."""
@@ -130,41 +108,6 @@ class Model(nn.Module):
             if self.trace_layers is not None:
                 self.trace_layers.append(x.clone())
         return x
-
-    def logits(self, x: torch.Tensor) -> torch.Tensor:
-        """Last norm and output head on rows of the stream."""
-        w = self.lm_head.weight
-        return F.linear(self.model.norm(x, w.dtype), w)
-
-    def _run(self, inputs: torch.Tensor, cache):
-        b, l = inputs.shape
-        if cache is None:
-            cache = self.make_cache()
-            for _ in range(b - 1):
-                cache[0].slots.acquire()
-        slots = cache[0].slots
-        if slots.n_slots < b or any(n < 0 for n in slots.length[:b]):
-            raise ValueError("the cache does not hold a sequence for every row of the batch")
-        batch = StepBatch.build(list(range(b)), [slots.length[s] for s in range(b)], [l] * b, inputs.device)
-        x = self.forward_tokens(inputs.reshape(-1), batch, cache)
-        for s in range(b):
-            slots.length[s] += l
-        return x
-
-    def forward(self, inputs: torch.Tensor, mask=None, cache=None, hidden_states: bool = False):
-        """[B, L] token ids, row b continuing sequence b of ``cache`` -> logits [B, L, vocab] (``generate_step`` convention)."""
-        b, l = inputs.shape
-        x = self._run(inputs, cache)
-        logits = self.logits(x).view(b, l, -1)
-        return (logits, x.view(b, l, -1)) if hidden_states else logits
-
-    def last_logits(self, inputs: torch.Tensor, cache) -> torch.Tensor:
-        """Logits of the last position only, [B, vocab]: the head never sees the prompt's other rows."""
-        b, l = inputs.shape
-        return self.logits(self._run(inputs, cache).view(b, l, -1)[:, -1])
-
-    def prefill(self, inputs: torch.Tensor, cache) -> None:
-        self._run(inputs, cache)
 
     def sanitize(self, weights: Dict[str, torch.Tensor]) -> Dict[str, torch.Tensor]:
         """Checkpoint names -> module paths.  q | k | v are concatenated into one projection, the experts stacked; norm weights,

@@ -151,3 +151,28 @@ def initialize_rope(dims, base, traditional, scaling_config: Optional[dict] = No
     if rope_type in ("yarn", "longrope"):
         raise NotImplementedError(f"RoPE type {rope_type} belongs to model families outside the Llama hot path")
     raise ValueError(f"Unsupported RoPE type {rope_type}")
+
+
+def rotary_table(base: float, dims: int, scaling: Optional[dict] = None):
+    """(frequencies fp32 [dims // 2], multiplier of cos and sin) of a rotation over ``dims`` channels with f_i = base^(-2i/dims).
+
+    ``scaling`` is None (plain), ``{"factor"}`` (linear: every frequency divided by the factor) or ``{"factor", "original", "fast",
+    "slow"}`` (YaRN: channels that turn more than ``fast`` times over the ``original`` context keep their frequency, channels that
+    turn less than ``slow`` times are divided by the factor, a linear ramp over the channel index between the two; cos and sin are
+    multiplied by 0.1 ln(factor) + 1).  Evaluated in float64 on the host, once per model."""
+    f = [base ** (-2.0 * i / dims) for i in range(dims // 2)]
+    mult = 1.0
+    if scaling:
+        factor = float(scaling["factor"])
+        if "original" in scaling:
+            def turn_dim(turns: float) -> float:
+                return dims * math.log(scaling["original"] / (2.0 * math.pi * turns)) / (2.0 * math.log(base))
+            lo = max(math.floor(turn_dim(scaling["fast"])), 0)
+            hi = min(math.ceil(turn_dim(scaling["slow"])), dims - 1)
+            for i in range(dims // 2):
+                ramp = min(max((i - lo) / max(hi - lo, 0.001), 0.0), 1.0)
+                f[i] = f[i] / factor * ramp + f[i] * (1.0 - ramp)
+            mult = 0.1 * math.log(factor) + 1.0
+        else:
+            f = [v / factor for v in f]
+    return torch.tensor(f, dtype=torch.float64).to(torch.float32), float(mult)

@@ -18,7 +18,7 @@ from typing import Any, Callable, Generator, List, Optional, Tuple, Type, Union
 import torch
 from torch import nn
 
-from .models import qdeepseek_v3, qllama, qmixtral, qphi3, qqwen2, qqwen3, qqwen3_moe, revitar
+from .models import qdeepseek_v3, qllama, qmixtral, qphi3, qqwen2, qqwen3, qqwen3_moe, radenex, revitar
 from .models import cache as cache_mod
 from .models.quantized_linear_gba import QuantizedLinear
 from .tokenizer_utils import TokenizerWrapper, load_tokenizer
@@ -32,6 +32,7 @@ MODEL_MAPPING = {
     "qwen2": qqwen2,
     "qwen3": qqwen3,
     "qwen3_moe": qqwen3_moe,
+    "radenex": radenex,       # dense checkpoint of parallel layers (latent / windowed sink attention), named by "architecture"
     "revitar": revitar,       # dense (unquantised) checkpoint; its config names itself by "architecture"
 }
 
