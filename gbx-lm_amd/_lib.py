@@ -309,6 +309,28 @@ class WindowAttnArgs(ctypes.Structure):
                 ("partial", ctypes.c_void_p), ("partial_splits", ctypes.c_int32)]
 
 
+class HeadSegment(ctypes.Structure):
+    """Mirror of ``gbxm_head_segment``."""
+    _fields_ = [("offset", ctypes.c_int32), ("heads", ctypes.c_int32), ("head_dim", ctypes.c_int32), ("rot_offset", ctypes.c_int32),
+                ("rot_dims", ctypes.c_int32), ("interleaved", ctypes.c_int32), ("norm", ctypes.c_int32), ("mult", ctypes.c_float),
+                ("sign", ctypes.c_float), ("freq", ctypes.c_void_p), ("weight", ctypes.c_void_p)]
+
+
+class SinkAttnArgs(ctypes.Structure):
+    """Mirror of ``gbxm_sink_attn_args``."""
+    _fields_ = [("q", ctypes.c_void_p), ("q_row", ctypes.c_int64), ("q_head", ctypes.c_int64),
+                ("k_new", ctypes.c_void_p), ("k_row", ctypes.c_int64), ("k_head", ctypes.c_int64),
+                ("v_new", ctypes.c_void_p), ("v_row", ctypes.c_int64), ("v_head", ctypes.c_int64),
+                ("kcache", ctypes.c_void_p), ("kc_slot", ctypes.c_int64), ("kc_row", ctypes.c_int64), ("kc_head", ctypes.c_int64),
+                ("vcache", ctypes.c_void_p), ("vc_slot", ctypes.c_int64), ("vc_row", ctypes.c_int64), ("vc_head", ctypes.c_int64),
+                ("seq", ctypes.c_void_p), ("tok", ctypes.c_void_p), ("tiles", ctypes.c_void_p), ("out", ctypes.c_void_p),
+                ("sink", ctypes.c_void_p), ("gate", ctypes.c_void_p), ("gate_row", ctypes.c_int64),
+                ("T", ctypes.c_int64), ("B", ctypes.c_int32), ("n_tiles", ctypes.c_int32), ("q_tile", ctypes.c_int32),
+                ("H", ctypes.c_int32), ("G", ctypes.c_int32), ("dk", ctypes.c_int32), ("dv", ctypes.c_int32),
+                ("window", ctypes.c_int32), ("keep", ctypes.c_int32), ("ring", ctypes.c_int32), ("scale", ctypes.c_float),
+                ("decode_only", ctypes.c_int32), ("act", ctypes.c_int32), ("partial", ctypes.c_void_p), ("partial_splits", ctypes.c_int32)]
+
+
 def mixers_so_path() -> str:
     return _MSO
 
@@ -346,6 +368,12 @@ def mixers() -> ctypes.CDLL:
         L.gbxm_window_attention.argtypes = [ctypes.POINTER(WindowAttnArgs), p]
         L.gbxm_window_attention_tiled.argtypes = [i32, i32, i32, i32]
         L.gbxm_window_append.argtypes = [p, i64, i32, i32, i32, p, p, p, p, i64, i32, i32, p]
+        L.gbxm_stream_add.argtypes = [p, p, p, i64, i32, p]
+        L.gbxm_activate.argtypes = [p, i64, i32, i32, p]
+        L.gbxm_rotate_norm_heads.argtypes = [p, i64, i64, p, i64, ctypes.POINTER(HeadSegment), i32, f32, i32, p]
+        L.gbxm_slot_append.argtypes = [p, i64, i32, p, i64, i32, p, p, p, p, i64, i32, i32, i32, p]
+        L.gbxm_sink_attention.argtypes = [ctypes.POINTER(SinkAttnArgs), p]
+        L.gbxm_sink_attention_tiled.argtypes = [i32, i32, i32, i32]
         _mlib = L
     return _mlib
 

@@ -180,6 +180,10 @@ class BatchScheduler:
 
     def _graph_step(self, slots: Tuple[int, ...], tokens: Sequence[int], pos0: Sequence[int]) -> Optional[torch.Tensor]:
         """Replay (or, at the third step of this set of slots, capture) the decode graph; None: run the step eagerly."""
+        longest = max(pos0) + 1
+        for c in self.caches:                            # tables without a window grow on the host, never inside a replay
+            if hasattr(c, "ensure"):
+                c.ensure(longest)
         buffers = tuple(c.keys.data_ptr() if c.keys is not None else 0 for c in self.caches)
         if buffers != self._buffers:                     # rings were (re)allocated: every captured pointer is stale
             self._graphs.clear()

@@ -202,7 +202,6 @@ const char* gbxm_last_error(void) { return g_err; }
 int gbxm_embed_scaled(const void* table, const int64_t* tokens, float* x, void* h, int64_t T_, int32_t width, float scale, int32_t act,
                       void* stream) {
   if (!act_ok(act) || !table || !tokens || !x || width <= 0 || T_ < 0) return fail(GBXM_ERR_INVALID, "embed_scaled: bad argument");
-  if (act == GBXM_BF16 && !h) return fail(GBXM_ERR_INVALID, "embed_scaled: bf16 needs the image buffer");
   if (T_ == 0) return GBXM_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
   GBXM_DISPATCH(act, (embed_kernel<T><<<dim3(T_), NT, 0, s>>>(static_cast<const T*>(table), tokens, x, static_cast<T*>(h), width, scale)));

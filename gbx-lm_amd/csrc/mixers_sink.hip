@@ -1,0 +1,464 @@
+// Softmax attention with a sink over a ragged step, and the row kernels around it: head rotations / norms, the append to slot
+// tables, the parallel-layer stream update and the feed-forward activation.
+//
+//   out[t][h] = gate[t][h] * sum_j p_j v_j,   p_j = exp(s_j) / (exp(sink_h) + sum_j exp(s_j)),   s_j = scale <q[t][h], k_j>
+// over the keys j <= i of the row's sequence with i - j < window or j < keep.  The keys a row sees are two runs of positions,
+// [0, min(keep, lo)) and [lo, i] with lo = max(0, i - window + 1); the kernels walk them as ONE run of indices (no masked key is
+// ever loaded).  Position j of a sequence is read from its slot's table (row j if j < keep, else keep + (j - keep) % ring) when it
+// lies before the step, and from the step's own rows otherwise.
+//
+// sink_rows_kernel: any head sizes, fp32 or bf16, all arithmetic fp32 -- one workgroup per (row, kv head, chunk of its query
+// heads, share of the key tiles); scores by a thread per (head, key) of a 64-key tile, running maximum / sum per head in LDS, the
+// value sum with a wave per key and the lanes across channels.  A step of few rows splits the key tiles over workgroups; each
+// leaves (sum, maximum, denominator) and sink_reduce_kernel joins them in a fixed order, adds the sink and applies the gate.
+// The matrix-core kernel for bf16 prompt portions is in mixers_sink_mfma.hip.
+#include <algorithm>
+#include <climits>
+#include "mixers_common.h"
+
+namespace gbxm {
+namespace {
+
+constexpr int NT = 256, NW = NT / 64;
+constexpr int KT = 64;            // keys per tile
+constexpr int RC = 8;             // query heads a workgroup takes at most
+constexpr int DCH = 128;          // value channels per lane pass (two per lane)
+constexpr int NCH = 4;            // lane passes: value sizes up to NCH * DCH
+
+struct SinkGeo {
+  int H, G, dk, dv, window, keep, ring;
+  float scale;
+  int64_t q_row, q_head, k_row, k_head, v_row, v_head, kc_slot, kc_row, kc_head, vc_slot, vc_row, vc_head, gate_row;
+};
+
+template <typename T, bool VEC>
+__device__ __forceinline__ float dot_row(const float* __restrict__ q, const T* __restrict__ k, int dk) {
+  float dot = 0.f;
+  if constexpr (VEC) {
+    constexpr int PER = 16 / sizeof(T);
+    for (int d = 0; d < dk; d += PER) {
+      const uint4 raw = *reinterpret_cast<const uint4*>(k + d);
+      if constexpr (sizeof(T) == 2) {
+        const unsigned u[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          dot += q[d + 2 * i] * __uint_as_float(u[i] << 16);
+          dot += q[d + 2 * i + 1] * __uint_as_float(u[i] & 0xFFFF0000u);
+        }
+      } else {
+        dot += q[d] * __uint_as_float(raw.x) + q[d + 1] * __uint_as_float(raw.y) + q[d + 2] * __uint_as_float(raw.z) + q[d + 3] * __uint_as_float(raw.w);
+      }
+    }
+  } else {
+    for (int d = 0; d < dk; ++d) dot += q[d] * to_f32(k[d]);
+  }
+  return dot;
+}
+
+template <typename T, bool FAST, bool VEC>
+__global__ __launch_bounds__(NT) void sink_rows_kernel(const T* __restrict__ q, const T* __restrict__ kn, const T* __restrict__ vn,
+                                                      const T* __restrict__ kc, const T* __restrict__ vc, const int* __restrict__ seq,
+                                                      const int* __restrict__ tok, T* __restrict__ out, const float* __restrict__ sink,
+                                                      const T* __restrict__ gate, SinkGeo g, int rc, int splits, float* __restrict__ partial) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  const T** kptr = reinterpret_cast<const T**>(lds_raw);            // [KT] rows of the tile's keys
+  const T** vptr = kptr + KT;                                        // [KT] and values
+  float* ql = reinterpret_cast<float*>(vptr + KT);                   // [rc][dk]
+  float* gl = ql + rc * g.dk;                                        // [rc][KT] scores, then weights
+  float* ml = gl + rc * KT;                                          // [rc] running maximum
+  float* ll = ml + rc;                                               // [rc] running denominator
+  float* al = ll + rc;                                               // [rc] rescale of this tile
+  float* sums = al + rc;                                             // [NW][rc * dv]
+  const int64_t t = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int R = g.H / g.G;
+  const int chunks = (R + rc - 1) / rc;
+  const int kvh = blockIdx.y / chunks, r0 = (blockIdx.y % chunks) * rc;
+  const int nr = min(rc, R - r0);                   // query heads of this workgroup: kvh * R + r0 + (0 .. nr-1)
+  const int b = tok[2 * t], pos = tok[2 * t + 1];
+  const int slot = seq[4 * b], pos0 = seq[4 * b + 1], row0 = seq[4 * b + 3];
+  const int head0 = kvh * R + r0;
+  for (int i = threadIdx.x; i < nr * g.dk; i += NT) ql[i] = to_f32(q[t * g.q_row + (head0 + i / g.dk) * g.q_head + i % g.dk]);
+  if (threadIdx.x < nr) {
+    const bool own_sink = sink && splits == 1;      // split key tiles: the sink joins in the reduce
+    ml[threadIdx.x] = own_sink ? sink[head0 + threadIdx.x] : -INFINITY;
+    ll[threadIdx.x] = own_sink ? 1.f : 0.f;
+  }
+  float acc[NCH][RC][2];
+#pragma unroll
+  for (int c = 0; c < NCH; ++c)
+#pragma unroll
+    for (int r = 0; r < RC; ++r) acc[c][r][0] = acc[c][r][1] = 0.f;
+  const bool pair_loads = g.dv % 2 == 0 && VEC;
+  // the visible keys as one run of indices: [0, na) are positions 0 .. na-1 (kept first tokens that left the window), the rest lo ..
+  const int lo = g.window > 0 ? max(0, pos - g.window + 1) : 0;
+  const int na = min(g.keep, lo);
+  const int total = na + (pos - lo + 1);
+  for (int it = static_cast<int>(blockIdx.z) * KT; it < total; it += KT * splits) {
+    __syncthreads();                                // the previous tile's weights and rows have been consumed
+    if (threadIdx.x < KT) {
+      const int iv = min(it + static_cast<int>(threadIdx.x), total - 1);
+      const int j = iv < na ? iv : lo + (iv - na);
+      if (j < pos0) {
+        const int64_t row = j < g.keep ? j : g.keep + (j - g.keep) % g.ring;
+        kptr[threadIdx.x] = kc + slot * g.kc_slot + row * g.kc_row + kvh * g.kc_head;
+        vptr[threadIdx.x] = vc + slot * g.vc_slot + row * g.vc_row + kvh * g.vc_head;
+      } else {
+        const int64_t row = row0 + (j - pos0);
+        kptr[threadIdx.x] = kn + row * g.k_row + kvh * g.k_head;
+        vptr[threadIdx.x] = vn + row * g.v_row + kvh * g.v_head;
+      }
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < nr * KT; i += NT) {
+      const int r = i / KT, jj = i % KT;
+      gl[i] = it + jj < total ? dot_row<T, VEC>(ql + r * g.dk, kptr[jj], g.dk) * g.scale : -INFINITY;
+    }
+    __syncthreads();
+    for (int r = wave; r < nr; r += NW) {           // a wave per head: the tile's maximum, the weights, their sum
+      const float s = gl[r * KT + lane];
+      float mx = s;
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+      const float m_old = ml[r], m_new = fmaxf(m_old, mx);            // mx is finite: a tile holds at least one key
+      const float p = exp_<FAST>(s - m_new);
+      gl[r * KT + lane] = p;
+      const float ps = wave_sum(p);
+      if (lane == 0) {
+        const float alpha = exp_<FAST>(m_old - m_new);                // exp(-inf) = 0 at the first tile without a sink
+        ml[r] = m_new; ll[r] = ll[r] * alpha + ps; al[r] = alpha;
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < RC; ++r)
+      if (r < nr) {
+        const float alpha = al[r];
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) { acc[c][r][0] *= alpha; acc[c][r][1] *= alpha; }
+      }
+    const int nj = min(KT, total - it);
+#pragma unroll 4
+    for (int jj = wave; jj < nj; jj += NW) {
+      const T* vr = vptr[jj];
+#pragma unroll
+      for (int c = 0; c < NCH; ++c) {
+        const int d0 = c * DCH + 2 * lane;
+        if (d0 < g.dv) {
+          float v0, v1 = 0.f;
+          if (pair_loads) {
+            if constexpr (sizeof(T) == 2) {
+              const unsigned u = *reinterpret_cast<const unsigned*>(vr + d0);
+              v0 = __uint_as_float(u << 16); v1 = __uint_as_float(u & 0xFFFF0000u);
+            } else {
+              const float2 f = *reinterpret_cast<const float2*>(vr + d0);
+              v0 = f.x; v1 = f.y;
+            }
+          } else {
+            v0 = to_f32(vr[d0]);
+            if (d0 + 1 < g.dv) v1 = to_f32(vr[d0 + 1]);
+          }
+#pragma unroll
+          for (int r = 0; r < RC; ++r)
+            if (r < nr) {
+              const float p = gl[r * KT + jj];
+              acc[c][r][0] += p * v0;
+              acc[c][r][1] += p * v1;
+            }
+        }
+      }
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int c = 0; c < NCH; ++c) {
+    const int d0 = c * DCH + 2 * lane;
+    if (d0 < g.dv)
+#pragma unroll
+      for (int r = 0; r < RC; ++r)
+        if (r < nr) {
+          sums[(wave * rc + r) * g.dv + d0] = acc[c][r][0];
+          if (d0 + 1 < g.dv) sums[(wave * rc + r) * g.dv + d0 + 1] = acc[c][r][1];
+        }
+  }
+  __syncthreads();
+  if (splits > 1) {
+    float* prow = partial + ((static_cast<int64_t>(blockIdx.z) * gridDim.x + t) * g.H + head0) * (g.dv + 2);
+    for (int i = threadIdx.x; i < nr * g.dv; i += NT) {
+      float s = 0.f;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) s += sums[w * rc * g.dv + i];
+      prow[(i / g.dv) * (g.dv + 2) + i % g.dv] = s;
+    }
+    if (threadIdx.x < nr) {
+      prow[threadIdx.x * (g.dv + 2) + g.dv] = ml[threadIdx.x];
+      prow[threadIdx.x * (g.dv + 2) + g.dv + 1] = ll[threadIdx.x];
+    }
+    return;
+  }
+  T* orow = out + t * (static_cast<int64_t>(g.H) * g.dv) + head0 * g.dv;
+  for (int i = threadIdx.x; i < nr * g.dv; i += NT) {
+    const int r = i / g.dv;
+    float s = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) s += sums[w * rc * g.dv + i];
+    s /= ll[r];
+    if (gate) s *= sigmoid_<FAST>(to_f32(gate[t * g.gate_row + head0 + r]));
+    orow[i] = from_f32<T>(s);
+  }
+}
+
+// One workgroup per (row, head): joins the key splits' (sum, maximum, denominator) in split order, adds the sink, applies the gate.
+template <typename T, bool FAST>
+__global__ __launch_bounds__(128) void sink_reduce_kernel(const float* __restrict__ partial, T* __restrict__ out, const float* __restrict__ sink,
+                                                         const T* __restrict__ gate, int64_t gate_row, int64_t T_, int H, int dv, int splits) {
+  __shared__ float wz[64];
+  __shared__ float den;
+  const int64_t t = blockIdx.x;
+  const int head = blockIdx.y;
+  const int64_t zs = T_ * H * (dv + 2);
+  const float* p0 = partial + (t * H + head) * (dv + 2);
+  if (threadIdx.x < 64) {
+    const int z = threadIdx.x;
+    const float m = z < splits ? p0[z * zs + dv] : -INFINITY;
+    float top = m;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) top = fmaxf(top, __shfl_xor(top, o, 64));
+    if (sink) top = fmaxf(top, sink[head]);
+    const float w = z < splits ? exp_<FAST>(m - top) : 0.f;
+    wz[z] = w;
+    float l = z < splits ? w * p0[z * zs + dv + 1] : 0.f;
+    l = wave_sum(l);
+    if (z == 0) den = l + (sink ? exp_<FAST>(sink[head] - top) : 0.f);
+  }
+  __syncthreads();
+  const float gv = gate ? sigmoid_<FAST>(to_f32(gate[t * gate_row + head])) : 1.f;
+  for (int d = threadIdx.x; d < dv; d += 128) {
+    float s = 0.f;
+    for (int z = 0; z < splits; ++z) s += wz[z] * p0[z * zs + d];
+    out[(t * H + head) * dv + d] = from_f32<T>(s / den * gv);
+  }
+}
+
+template <typename T, bool FAST>
+int launch_rows(const gbxm_sink_attn_args& a, const SinkGeo& g, int rc, int chunks, size_t lds, hipStream_t s) {
+  constexpr int PER = 16 / sizeof(T);
+  auto al = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+  bool vec = a.dk % PER == 0 && a.k_row % PER == 0 && a.k_head % PER == 0 && al(a.k_new) && a.v_row % 2 == 0 && a.v_head % 2 == 0 &&
+             reinterpret_cast<uintptr_t>(a.v_new) % 8 == 0;
+  if (a.kcache)
+    vec = vec && a.kc_slot % PER == 0 && a.kc_row % PER == 0 && a.kc_head % PER == 0 && al(a.kcache) && a.vc_slot % 2 == 0 && a.vc_row % 2 == 0 &&
+          a.vc_head % 2 == 0 && reinterpret_cast<uintptr_t>(a.vcache) % 8 == 0;
+  int splits = 1;
+  const int64_t groups = a.T * a.G * chunks;
+  if (a.partial && a.partial_splits > 1 && groups < 256) {
+    splits = static_cast<int>(std::min<int64_t>(std::min<int64_t>(512 / groups, 64), a.partial_splits));
+    if (splits < 2) splits = 1;
+  }
+  const dim3 grid(a.T, a.G * chunks, splits);
+  const T* q = static_cast<const T*>(a.q);
+  const T* kn = static_cast<const T*>(a.k_new);
+  const T* vn = static_cast<const T*>(a.v_new);
+  const T* kc = static_cast<const T*>(a.kcache);
+  const T* vc = static_cast<const T*>(a.vcache);
+  const T* gate = static_cast<const T*>(a.gate);
+  T* out = static_cast<T*>(a.out);
+  float* part = static_cast<float*>(a.partial);
+  if (vec)
+    sink_rows_kernel<T, FAST, true><<<grid, NT, lds, s>>>(q, kn, vn, kc, vc, a.seq, a.tok, out, a.sink, gate, g, rc, splits, part);
+  else
+    sink_rows_kernel<T, FAST, false><<<grid, NT, lds, s>>>(q, kn, vn, kc, vc, a.seq, a.tok, out, a.sink, gate, g, rc, splits, part);
+  if (splits > 1) sink_reduce_kernel<T, FAST><<<dim3(a.T, a.H), 128, 0, s>>>(part, out, a.sink, gate, a.gate_row, a.T, a.H, a.dv, splits);
+  return after_launch("sink_attention (rows)");
+}
+
+// ------------------------------------------------------------------------------------------------ rotations and norms of heads
+struct Segments {
+  gbxm_head_segment s[GBXM_MAX_SEGMENTS];
+};
+
+// One workgroup per (row, segment); its waves take the segment's heads four at a time.  A head is staged in LDS as fp32, every
+// lane forms its rotated channels from there (its own and the partner of the pair), the statistic is a wave sum.
+template <typename T>
+__global__ __launch_bounds__(NT) void rotate_norm_kernel(T* __restrict__ rows, int64_t stride, const int* __restrict__ positions, int64_t pos_stride,
+                                                        Segments segs, float eps, int max_dim) {
+  extern __shared__ float head_lds[];               // [NW][2][max_dim]
+  const gbxm_head_segment sg = segs.s[blockIdx.y];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  float* in = head_lds + wave * 2 * max_dim;
+  float* turned = in + max_dim;
+  const float pos = static_cast<float>(positions[blockIdx.x * pos_stride]);
+  const int half = sg.rot_dims / 2;
+  for (int h0 = 0; h0 < sg.heads; h0 += NW) {
+    const int head = h0 + wave;
+    const bool live = head < sg.heads;
+    T* p = rows + blockIdx.x * stride + sg.offset + static_cast<int64_t>(live ? head : 0) * sg.head_dim;
+    __syncthreads();
+    if (live)
+      for (int c = lane; c < sg.head_dim; c += 64) in[c] = to_f32(p[c]);
+    __syncthreads();
+    if (!live) continue;
+    float ss = 0.f;
+    for (int c = lane; c < sg.head_dim; c += 64) {
+      float v = in[c];
+      const int idx = c - sg.rot_offset;
+      if (idx >= 0 && idx < sg.rot_dims) {
+        int i, other;
+        bool first;
+        if (sg.interleaved) { i = idx >> 1; first = !(idx & 1); other = first ? c + 1 : c - 1; }
+        else { first = idx < half; i = first ? idx : idx - half; other = first ? c + half : c - half; }
+        float sn, cs;
+        sincosf(pos * sg.freq[i], &sn, &cs);
+        sn *= sg.mult * sg.sign; cs *= sg.mult;
+        // (u, w) -> (u cos - w sin, w cos + u sin)
+        v = first ? v * cs - in[other] * sn : v * cs + in[other] * sn;
+      }
+      turned[c] = v;
+      ss += v * v;
+    }
+    float r = 1.f;
+    if (sg.norm) r = 1.f / sqrtf(wave_sum(ss) / sg.head_dim + eps);
+    for (int c = lane; c < sg.head_dim; c += 64) {
+      float v = turned[c] * r;
+      if (sg.norm == 2) v *= sg.weight[c];
+      p[c] = from_f32<T>(v);
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(NT) void stream_add_kernel(float* __restrict__ x, const T* __restrict__ a, const T* __restrict__ b, int64_t n) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * NT + threadIdx.x;
+  if (i >= n) return;
+  float y = to_f32(a[i]);
+  if (b) y += to_f32(b[i]);
+  x[i] += y;
+}
+
+template <typename T>
+__global__ __launch_bounds__(NT) void activate_kernel(T* __restrict__ z, int64_t n, int kind) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * NT + threadIdx.x;
+  if (i >= n) return;
+  const float v = to_f32(z[i]);
+  float y;
+  if (kind == GBXM_ACT_RELU2) { const float r = fmaxf(v, 0.f); y = r * r; }
+  else y = 0.5f * v * (1.f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
+  z[i] = from_f32<T>(y);
+}
+
+template <typename T>
+__global__ __launch_bounds__(NT) void slot_append_kernel(const T* __restrict__ k, int64_t k_stride, int k_width, const T* __restrict__ v,
+                                                        int64_t v_stride, int v_width, T* __restrict__ kc, T* __restrict__ vc,
+                                                        const int* __restrict__ seq, const int* __restrict__ tok, int keep, int ring) {
+  const int64_t t = blockIdx.x;
+  const int b = tok[2 * t], pos = tok[2 * t + 1];
+  const int slot = seq[4 * b], pos0 = seq[4 * b + 1], n = seq[4 * b + 2];
+  if (pos >= keep && pos + ring < pos0 + n) return;      // a later row of this step takes the same ring row
+  const int64_t row = static_cast<int64_t>(slot) * (keep + ring) + (pos < keep ? pos : keep + (pos - keep) % ring);
+  for (int c = threadIdx.x; c < k_width; c += NT) kc[row * k_width + c] = k[t * k_stride + c];
+  if (v)
+    for (int c = threadIdx.x; c < v_width; c += NT) vc[row * v_width + c] = v[t * v_stride + c];
+}
+
+bool act_ok(int act) { return act == GBXM_BF16 || act == GBXM_F32; }
+
+}  // namespace
+
+int launch_sink_tiles(const gbxm_sink_attn_args& a, hipStream_t s);     // mixers_sink_mfma.hip; GBXM_ERR_UNSUPPORTED: not its shape
+bool sink_tiles_shape(int dk, int dv);
+
+}  // namespace gbxm
+
+using namespace gbxm;
+
+#define GBXM_DISPATCH(act, CALL)              \
+  do {                                        \
+    if ((act) == GBXM_BF16) { using T = bf16_t; CALL; } else { using T = float; CALL; } \
+  } while (0)
+
+extern "C" {
+
+int gbxm_stream_add(float* x, const void* a, const void* b, int64_t n, int32_t act, void* stream) {
+  if (!act_ok(act) || !x || !a || n < 0) return fail(GBXM_ERR_INVALID, "stream_add: bad argument");
+  if (n == 0) return GBXM_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  GBXM_DISPATCH(act, (stream_add_kernel<T><<<dim3((n + NT - 1) / NT), NT, 0, s>>>(x, static_cast<const T*>(a), static_cast<const T*>(b), n)));
+  return after_launch("stream_add");
+}
+
+int gbxm_activate(void* z, int64_t n, int32_t kind, int32_t act, void* stream) {
+  if (!act_ok(act) || !z || n < 0 || (kind != GBXM_ACT_RELU2 && kind != GBXM_ACT_GELU_TANH)) return fail(GBXM_ERR_INVALID, "activate: bad argument");
+  if (n == 0) return GBXM_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  GBXM_DISPATCH(act, (activate_kernel<T><<<dim3((n + NT - 1) / NT), NT, 0, s>>>(static_cast<T*>(z), n, kind)));
+  return after_launch("activate");
+}
+
+int gbxm_rotate_norm_heads(void* rows, int64_t T_, int64_t row_stride, const int32_t* positions, int64_t pos_stride, const gbxm_head_segment* segs,
+                           int32_t n_segs, float eps, int32_t act, void* stream) {
+  if (!act_ok(act) || !rows || !positions || !segs || n_segs < 1 || n_segs > GBXM_MAX_SEGMENTS || T_ < 0)
+    return fail(GBXM_ERR_INVALID, "rotate_norm_heads: bad argument");
+  Segments sg{};
+  int max_dim = 0;
+  for (int i = 0; i < n_segs; ++i) {
+    const gbxm_head_segment& g = segs[i];
+    if (g.offset < 0 || g.heads < 1 || g.head_dim < 1 || g.offset + static_cast<int64_t>(g.heads) * g.head_dim > row_stride || g.rot_dims < 0 ||
+        g.rot_dims % 2 || g.rot_offset < 0 || g.rot_offset + g.rot_dims > g.head_dim || (g.rot_dims && !g.freq) || g.norm < 0 || g.norm > 2 ||
+        (g.norm == 2 && !g.weight))
+      return fail(GBXM_ERR_INVALID, "rotate_norm_heads: segment %d does not fit its rows", i);
+    sg.s[i] = g;
+    max_dim = std::max(max_dim, g.head_dim);
+  }
+  const size_t lds = static_cast<size_t>(NW) * 2 * max_dim * sizeof(float);
+  if (lds > 60 * 1024) return fail(GBXM_ERR_UNSUPPORTED, "rotate_norm_heads: heads of %d channels", max_dim);
+  if (T_ == 0) return GBXM_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  GBXM_DISPATCH(act, (rotate_norm_kernel<T><<<dim3(T_, n_segs), NT, lds, s>>>(static_cast<T*>(rows), row_stride, positions, pos_stride, sg, eps, max_dim)));
+  return after_launch("rotate_norm_heads");
+}
+
+int gbxm_slot_append(const void* k, int64_t k_stride, int32_t k_width, const void* v, int64_t v_stride, int32_t v_width, void* kcache, void* vcache,
+                     const int32_t* seq, const int32_t* tok, int64_t T_, int32_t keep, int32_t ring, int32_t act, void* stream) {
+  if (!act_ok(act) || !k || !kcache || !seq || !tok || k_width <= 0 || k_stride < k_width || keep < 0 || ring < 1 || T_ < 0 ||
+      (v && (!vcache || v_width <= 0 || v_stride < v_width)))
+    return fail(GBXM_ERR_INVALID, "slot_append: bad argument");
+  if (T_ == 0) return GBXM_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  GBXM_DISPATCH(act, (slot_append_kernel<T><<<dim3(T_), NT, 0, s>>>(static_cast<const T*>(k), k_stride, k_width, static_cast<const T*>(v), v_stride,
+                                                                      v_width, static_cast<T*>(kcache), static_cast<T*>(vcache), seq, tok, keep, ring)));
+  return after_launch("slot_append");
+}
+
+int gbxm_sink_attention_tiled(int32_t dk, int32_t dv, int32_t act, int32_t decode_only) {
+  return act == GBXM_BF16 && !decode_only && sink_tiles_shape(dk, dv);
+}
+
+int gbxm_sink_attention(const gbxm_sink_attn_args* a, void* stream) {
+  if (!a || !a->q || !a->k_new || !a->v_new || !a->seq || !a->tok || !a->out) return fail(GBXM_ERR_INVALID, "sink_attention: null argument");
+  if (!act_ok(a->act)) return fail(GBXM_ERR_INVALID, "sink_attention: dtype");
+  if (a->H <= 0 || a->G <= 0 || a->H % a->G || a->dk <= 0 || a->dv <= 0 || a->keep < 0 || a->ring < 1 || a->T < 0 || a->B < 0 ||
+      (a->kcache && !a->vcache))
+    return fail(GBXM_ERR_INVALID, "sink_attention: bad geometry");
+  if (a->window > 0 && a->ring < a->window) return fail(GBXM_ERR_INVALID, "sink_attention: a ring shorter than the window");
+  if (a->T == 0) return GBXM_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (!a->decode_only && a->act == GBXM_BF16 && a->tiles && a->n_tiles > 0) {
+    const int rc = launch_sink_tiles(*a, s);
+    if (rc != GBXM_ERR_UNSUPPORTED) return rc;
+  }
+  SinkGeo g{a->H, a->G, a->dk, a->dv, a->window, a->keep, a->ring, a->scale, a->q_row, a->q_head, a->k_row, a->k_head, a->v_row, a->v_head,
+            a->kc_slot, a->kc_row, a->kc_head, a->vc_slot, a->vc_row, a->vc_head, a->gate_row};
+  const int R = a->H / a->G;
+  if (a->dv > NCH * DCH) return fail(GBXM_ERR_UNSUPPORTED, "sink_attention: value size %d beyond the row kernel (%d)", a->dv, NCH * DCH);
+  auto lds_of = [&](int rc_) {
+    return static_cast<size_t>(2 * KT) * sizeof(void*) + static_cast<size_t>(rc_) * (a->dk + KT + 3 + NW * a->dv) * sizeof(float);
+  };
+  int rc = R < RC ? R : RC;
+  while (rc > 1 && lds_of(rc) > 60 * 1024) --rc;
+  if (lds_of(rc) > 60 * 1024) return fail(GBXM_ERR_UNSUPPORTED, "sink_attention: head sizes dk=%d dv=%d are beyond the row kernel", a->dk, a->dv);
+  const int chunks = (R + rc - 1) / rc;
+  if (a->T > 0x7fffffffLL || a->G * chunks > 65535 || a->H > 65535) return fail(GBXM_ERR_UNSUPPORTED, "sink_attention: grid");
+  return a->act == GBXM_BF16 ? launch_rows<bf16_t, true>(*a, g, rc, chunks, lds_of(rc), s) : launch_rows<float, false>(*a, g, rc, chunks, lds_of(rc), s);
+}
+
+}  // extern "C"

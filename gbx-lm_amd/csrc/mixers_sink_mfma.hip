@@ -1,0 +1,218 @@
+// Matrix-core kernel of softmax attention with a sink for bf16 prompt portions (mechanism and key order: mixers_sink.hip).
+//
+// One workgroup = 4 waves = one tile of up to 128 query rows of one (sequence, head); a wave owns 32 queries.  Key / value tiles
+// of 32 visible positions go global -> registers (one tile ahead) -> LDS once per workgroup.  Both products are computed swapped,
+//   S^T[key, q] = mfma(K rows, Q rows),    O^T[d, q] += mfma(V^T rows, P^T),
+// so that a lane owns ONE query: lane (q = lane % 32, half = lane / 32) holds 16 of the tile's 32 scores of its query, the other 16
+// are in lane ^ 32.  The running maximum is shared by the two lanes of a query (one cross-lane exchange per tile), each keeps its
+// own part of the denominator (joined once at the end), and both rescale their accumulators (different channels of the same
+// query) by the same factor.  The sink starts the running maximum and counts once in the denominator.  Weights are rounded to bf16
+// for the value product; the denominator sums them in fp32.
+//
+// Head sizes are run-time numbers (multiples of 8) inside a compiled capacity <DK, DV>: channels beyond them are staged as zeros.
+#include "mixers_mfma.h"
+
+namespace gbxm {
+namespace {
+
+struct SinkTileArgs {
+  const bf16_t* q;
+  const bf16_t* kn;
+  const bf16_t* vn;
+  const bf16_t* kc;
+  const bf16_t* vc;
+  const int* seq;
+  const int* tiles;
+  bf16_t* out;
+  const float* sink;
+  const bf16_t* gate;
+  int64_t q_row, q_head, k_row, k_head, v_row, v_head, kc_slot, kc_row, kc_head, vc_slot, vc_row, vc_head, gate_row;
+  int q_tile, H, G, dk, dv, window, keep, ring;
+  float scale;
+};
+
+template <int DK, int DV>
+__global__ __launch_bounds__(256) void sink_tile_kernel(const SinkTileArgs a) {
+  constexpr int KT = 32;
+  constexpr int KROW = DK * 2 + 16;          // +16 B: conflict-free 16-byte fragment reads
+  constexpr int VROW = DV * 2 + 64;          // pitch = 16 dwords mod 64: the 4 rows of a transposed block land on disjoint banks
+  constexpr int KS = DK / 16, DT = DV / 32;
+  __shared__ __attribute__((aligned(16))) unsigned char lds[KT * KROW + KT * VROW];
+  unsigned char* kl = lds;
+  unsigned char* vl = lds + KT * KROW;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 31, hb = lane >> 5;
+  const int b = a.tiles[2 * blockIdx.x], tq = a.tiles[2 * blockIdx.x + 1];
+  const int head = blockIdx.y, kvh = head / (a.H / a.G);
+  const int slot = a.seq[4 * b], pos0 = a.seq[4 * b + 1], n = a.seq[4 * b + 2], row0 = a.seq[4 * b + 3];
+  const int W = a.window;
+  const int qn = min(a.q_tile, n - tq);                     // queries of this tile
+  const int qloc = wave * 32 + r;
+  const bool qvalid = qloc < qn;
+  const int qpos = pos0 + tq + qloc;
+
+  u32x4 qf[KS];
+  {
+    const bf16_t* qp = a.q + (row0 + tq + min(qloc, qn - 1)) * a.q_row + head * a.q_head;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int c = ks * 16 + hb * 8;
+      qf[ks] = c < a.dk ? *reinterpret_cast<const u32x4*>(qp + c) : u32x4{0, 0, 0, 0};
+    }
+  }
+  f32x16 o[DT];
+#pragma unroll
+  for (int i = 0; i < DT; ++i) o[i] = f32x16{0};
+
+  // the keys any query of the tile sees, as one run of indices: [0, na) are positions 0 .. na-1, the rest lo .. jlast
+  const int qfirst = pos0 + tq, jlast = qfirst + qn - 1;
+  const int lo = W > 0 ? max(0, qfirst - W + 1) : 0;
+  const int na = min(a.keep, lo);
+  const int total = na + (jlast - lo + 1);
+  auto pos_of = [&](int iv) { return iv < na ? iv : lo + (iv - na); };
+  const bool wave_live = wave * 32 < qn;
+  const int wq0 = qfirst + wave * 32, wq1 = min(wq0 + 31, jlast);      // positions of this wave's queries
+
+  float m = a.sink ? a.sink[head] : -INFINITY;
+  float l = (a.sink && hb == 0) ? 1.f : 0.f;                            // the sink counts once per query
+  const float scale = a.scale;
+  const unsigned char* vbase = vl + (4 * hb + ((lane >> 2) & 3)) * VROW + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
+  const unsigned char* kbase = kl + r * KROW + hb * 16;
+
+  auto krow = [&](int j) -> const bf16_t* {
+    if (j < pos0) return a.kc + slot * a.kc_slot + static_cast<int64_t>(j < a.keep ? j : a.keep + (j - a.keep) % a.ring) * a.kc_row + kvh * a.kc_head;
+    return a.kn + static_cast<int64_t>(row0 + (j - pos0)) * a.k_row + kvh * a.k_head;
+  };
+  auto vrow = [&](int j) -> const bf16_t* {
+    if (j < pos0) return a.vc + slot * a.vc_slot + static_cast<int64_t>(j < a.keep ? j : a.keep + (j - a.keep) % a.ring) * a.vc_row + kvh * a.vc_head;
+    return a.vn + static_cast<int64_t>(row0 + (j - pos0)) * a.v_row + kvh * a.v_head;
+  };
+
+  constexpr int KP = (KT * (DK / 8) + 255) / 256, VP = (KT * (DV / 8) + 255) / 256;
+  u32x4 kr[KP], vr[VP];
+  auto fetch = [&](int it) {
+#pragma unroll
+    for (int i = 0; i < KP; ++i) {
+      const int p = tid + 256 * i, row = p / (DK / 8), c = p % (DK / 8), iv = it + row;
+      kr[i] = u32x4{0, 0, 0, 0};
+      if (p < KT * (DK / 8) && iv < total && c * 8 < a.dk) kr[i] = *reinterpret_cast<const u32x4*>(krow(pos_of(iv)) + c * 8);
+    }
+#pragma unroll
+    for (int i = 0; i < VP; ++i) {
+      const int p = tid + 256 * i, row = p / (DV / 8), c = p % (DV / 8), iv = it + row;
+      vr[i] = u32x4{0, 0, 0, 0};
+      if (p < KT * (DV / 8) && iv < total && c * 8 < a.dv) vr[i] = *reinterpret_cast<const u32x4*>(vrow(pos_of(iv)) + c * 8);
+    }
+  };
+  fetch(0);
+  for (int it = 0; it < total; it += KT) {
+    __syncthreads();                                          // the previous tile has been consumed
+#pragma unroll
+    for (int i = 0; i < KP; ++i) {
+      const int p = tid + 256 * i;
+      if (p < KT * (DK / 8)) *reinterpret_cast<u32x4*>(kl + (p / (DK / 8)) * KROW + (p % (DK / 8)) * 16) = kr[i];
+    }
+#pragma unroll
+    for (int i = 0; i < VP; ++i) {
+      const int p = tid + 256 * i;
+      if (p < KT * (DV / 8)) *reinterpret_cast<u32x4*>(vl + (p / (DV / 8)) * VROW + (p % (DV / 8)) * 16) = vr[i];
+    }
+    __syncthreads();
+    if (it + KT < total) fetch(it + KT);                      // the next tile travels while this one is computed
+    // wave-uniform: no key of the tile is seen by a query of this wave
+    const int jmin = pos_of(it), jmax = pos_of(min(it + KT, total) - 1);
+    if (!wave_live || jmin > wq1 || (W > 0 && jmax < wq0 - W + 1 && jmin >= a.keep)) continue;
+
+    f32x16 st = f32x16{0};
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) st = mfma_bf16(*reinterpret_cast<const u32x4*>(kbase + ks * 32), qf[ks], st);
+    float s[16];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const int iv = it + 8 * (e >> 2) + 4 * hb + (e & 3);
+      const int j = pos_of(iv);
+      const bool seen = qvalid && iv < total && j <= qpos && (W <= 0 || qpos - j < W || j < a.keep);
+      s[e] = seen ? st[e] * scale : -INFINITY;
+      mx = fmaxf(mx, s[e]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));                   // the other half of the query's scores
+    const float m_new = fmaxf(m, mx);
+    const float m_ref = m_new == -INFINITY ? 0.f : m_new;     // nothing seen yet and no sink: every weight below is exp(-inf) = 0
+    const float alpha = __expf(m - m_ref);
+    m = m_new;
+    float ps = 0.f;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) { s[e] = __expf(s[e] - m_ref); ps += s[e]; }
+    l = l * alpha + ps;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) o[dt][e] *= alpha;
+    u32x4 gf[2];
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt)
+      gf[tt] = u32x4{pack2(s[8 * tt], s[8 * tt + 1]), pack2(s[8 * tt + 2], s[8 * tt + 3]), pack2(s[8 * tt + 4], s[8 * tt + 5]),
+                     pack2(s[8 * tt + 6], s[8 * tt + 7])};
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt) {
+        const u32x2 v0 = lds_read_tr(vbase + (16 * tt) * VROW + dt * 64);
+        const u32x2 v1 = lds_read_tr(vbase + (16 * tt + 8) * VROW + dt * 64);
+        o[dt] = mfma_bf16(u32x4{v0.x, v0.y, v1.x, v1.y}, gf[tt], o[dt]);
+      }
+  }
+
+  l += __shfl_xor(l, 32, 64);
+  if (qvalid) {
+    const int64_t row = row0 + tq + qloc;
+    float f = 1.f / l;
+    if (a.gate) f *= sigmoid_<true>(to_f32(a.gate[row * a.gate_row + head]));
+    bf16_t* op = a.out + row * (static_cast<int64_t>(a.H) * a.dv) + head * a.dv;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const int d = dt * 32 + 8 * q4 + 4 * hb;
+        if (d < a.dv)                                          // dv is a multiple of 8: the four channels are inside together
+          *reinterpret_cast<u32x2*>(op + d) = u32x2{pack2(o[dt][4 * q4] * f, o[dt][4 * q4 + 1] * f), pack2(o[dt][4 * q4 + 2] * f, o[dt][4 * q4 + 3] * f)};
+      }
+  }
+}
+
+template <int DK, int DV>
+int launch(const SinkTileArgs& t, int n_tiles, hipStream_t s) {
+  sink_tile_kernel<DK, DV><<<dim3(n_tiles, t.H), 256, 0, s>>>(t);
+  return after_launch("sink_attention (tiles)");
+}
+
+constexpr int CAPS[][2] = {{32, 32}, {64, 64}, {64, 128}, {96, 96}, {128, 128}, {192, 128}, {256, 256}};
+
+}  // namespace
+
+bool sink_tiles_shape(int dk, int dv) {
+  if (dk % 8 || dv % 8) return false;
+  for (const auto& c : CAPS)
+    if (dk <= c[0] && dv <= c[1]) return true;
+  return false;
+}
+
+int launch_sink_tiles(const gbxm_sink_attn_args& a, hipStream_t s) {
+  if (!sink_tiles_shape(a.dk, a.dv) || a.q_tile != 128 || a.H > 65535) return GBXM_ERR_UNSUPPORTED;
+  auto al = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+  if ((a.q_row | a.q_head | a.k_row | a.k_head | a.v_row | a.v_head) % 8 || !al(a.q) || !al(a.k_new) || !al(a.v_new) || !al(a.out))
+    return GBXM_ERR_UNSUPPORTED;
+  if (a.kcache && ((a.kc_slot | a.kc_row | a.kc_head | a.vc_slot | a.vc_row | a.vc_head) % 8 || !al(a.kcache) || !al(a.vcache))) return GBXM_ERR_UNSUPPORTED;
+  SinkTileArgs t{static_cast<const bf16_t*>(a.q), static_cast<const bf16_t*>(a.k_new), static_cast<const bf16_t*>(a.v_new),
+                 static_cast<const bf16_t*>(a.kcache), static_cast<const bf16_t*>(a.vcache), a.seq, a.tiles, static_cast<bf16_t*>(a.out), a.sink,
+                 static_cast<const bf16_t*>(a.gate), a.q_row, a.q_head, a.k_row, a.k_head, a.v_row, a.v_head, a.kc_slot, a.kc_row, a.kc_head,
+                 a.vc_slot, a.vc_row, a.vc_head, a.gate_row, a.q_tile, a.H, a.G, a.dk, a.dv, a.window, a.keep, a.ring, a.scale};
+#define GBXM_TILE(DK_, DV_) if (a.dk <= DK_ && a.dv <= DV_) return launch<DK_, DV_>(t, a.n_tiles, s)
+  GBXM_TILE(32, 32); GBXM_TILE(64, 64); GBXM_TILE(64, 128); GBXM_TILE(96, 96); GBXM_TILE(128, 128); GBXM_TILE(192, 128); GBXM_TILE(256, 256);
+#undef GBXM_TILE
+  return GBXM_ERR_UNSUPPORTED;
+}
+
+}  // namespace gbxm

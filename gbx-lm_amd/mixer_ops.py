@@ -1,6 +1,7 @@
 """Operator wrappers of libgbx_mixers.so: torch tensors in, raw device pointers across the C-ABI (include/gbx_mixers.h).
 
-These are the GPU halves of models/window_attention.py, models/switch_layers.py:DenseRoutedGLU and models/residual.py; each takes
+These are the GPU halves of models/window_attention.py, models/sink_attention.py, models/switch_layers.py:DenseRoutedGLU,
+models/feed_forward.py and models/residual.py; each takes
 rows of a ragged step (batching.StepBatch).  CPU tensors are refused: the modules run their plain torch graph for those.
 """
 from __future__ import annotations
@@ -33,13 +34,14 @@ def _f32(t: torch.Tensor, name: str) -> torch.Tensor:
     return t
 
 
-def embed_scaled(table: torch.Tensor, tokens: torch.Tensor, scale: float):
-    """(x fp32 [T, W], h in the table's dtype): x = table[tokens] * scale; h is x itself for an fp32 table."""
+def embed_scaled(table: torch.Tensor, tokens: torch.Tensor, scale: float, image: bool = True):
+    """(x fp32 [T, W], h in the table's dtype): x = table[tokens] * scale; h is x itself for an fp32 table or when no image is asked
+    for (a model whose first layer norms the stream itself)."""
     act = _act(table, "table")
     t, w = tokens.numel(), table.shape[1]
     tokens = tokens.reshape(-1).to(torch.long).contiguous()
     x = torch.empty((t, w), dtype=torch.float32, device=table.device)
-    h = x if table.dtype == torch.float32 else torch.empty((t, w), dtype=table.dtype, device=table.device)
+    h = x if (table.dtype == torch.float32 or not image) else torch.empty((t, w), dtype=table.dtype, device=table.device)
     _lib.check_mixers(_lib.mixers().gbxm_embed_scaled(table.data_ptr(), tokens.data_ptr(), x.data_ptr(), None if h is x else h.data_ptr(),
                                                      t, w, float(scale), act, _stream(table.device)))
     return x, h
@@ -147,3 +149,117 @@ def window_append(qkv: torch.Tensor, nq: int, nk: int, kcache: torch.Tensor, vca
     nv = qkv.shape[1] - nq - nk
     _lib.check_mixers(_lib.mixers().gbxm_window_append(qkv.data_ptr(), qkv.stride(0), nq, nk, nv, kcache.data_ptr(), vcache.data_ptr(),
                                                       batch.seq.data_ptr(), batch.tok.data_ptr(), batch.total, window, act, _stream(qkv.device)))
+
+
+# ------------------------------------------------------------------------------- softmax attention with a sink and its row kernels
+def stream_add_(x: torch.Tensor, a: torch.Tensor, b: Optional[torch.Tensor] = None) -> torch.Tensor:
+    act = _act(a, "a")
+    _f32(x, "x")
+    if a.shape != x.shape or not a.is_contiguous() or (b is not None and (b.shape != x.shape or b.dtype != a.dtype or not b.is_contiguous())):
+        raise ValueError("stream_add_: contiguous branches of the stream's shape and one dtype")
+    _lib.check_mixers(_lib.mixers().gbxm_stream_add(x.data_ptr(), a.data_ptr(), None if b is None else b.data_ptr(), x.numel(), act,
+                                                   _stream(x.device)))
+    return x
+
+
+_ACTIVATION = {"relu2": 1, "gelu_tanh": 2}
+
+
+def activate_(z: torch.Tensor, kind: str) -> torch.Tensor:
+    act = _act(z, "z")
+    if not z.is_contiguous():
+        raise ValueError("activate_: contiguous rows")
+    _lib.check_mixers(_lib.mixers().gbxm_activate(z.data_ptr(), z.numel(), _ACTIVATION[kind], act, _stream(z.device)))
+    return z
+
+
+def rotate_norm_heads_(rows: torch.Tensor, positions: torch.Tensor, segments, eps: float) -> None:
+    """In place on rows [T, N] (unit inner stride): each ``HeadSegment`` (models/sink_attention.py) rotated and / or normalised."""
+    act = _act(rows, "rows")
+    if rows.dim() != 2 or rows.stride(1) != 1 or positions.dtype != torch.int32 or positions.dim() != 1 or positions.shape[0] != rows.shape[0]:
+        raise ValueError("rotate_norm_heads_: rows [T, N] with unit inner stride and int32 positions [T]")
+    segs = (_lib.HeadSegment * len(segments))()
+    for c, s in zip(segs, segments):
+        if s.offset + s.heads * s.head_dim > rows.shape[1]:
+            raise ValueError("rotate_norm_heads_: a segment ends outside the rows")
+        if s.rot_dims and s.freq.numel() != s.rot_dims // 2:
+            raise ValueError("rotate_norm_heads_: one frequency per rotated pair")
+        if s.weight is not None and s.weight.numel() != s.head_dim:
+            raise ValueError("rotate_norm_heads_: one weight per channel of the head")
+        c.offset, c.heads, c.head_dim, c.rot_offset, c.rot_dims = s.offset, s.heads, s.head_dim, s.rot_offset, s.rot_dims
+        c.interleaved, c.norm, c.mult, c.sign = int(s.interleaved), s.norm, s.mult, s.sign
+        c.freq = _f32(s.freq, "freq").data_ptr() if s.rot_dims else None
+        c.weight = _f32(s.weight, "weight").data_ptr() if s.weight is not None else None
+    _lib.check_mixers(_lib.mixers().gbxm_rotate_norm_heads(rows.data_ptr(), rows.shape[0], rows.stride(0), positions.data_ptr(), positions.stride(0),
+                                                          segs, len(segments), float(eps), act, _stream(rows.device)))
+
+
+def slot_append(cache, k_rows: torch.Tensor, v_rows: Optional[torch.Tensor], batch) -> None:
+    act = _act(k_rows, "k_rows")
+    if k_rows.stride(1) != 1 or k_rows.shape[1] != cache.k_width or cache.keys.dtype != k_rows.dtype or cache.keys.shape[0] <= max(batch.slot):
+        raise ValueError("slot_append: key rows do not fit the table")
+    two = v_rows is not None
+    if two != bool(cache.v_width) or (two and (v_rows.stride(1) != 1 or v_rows.shape[1] != cache.v_width)):
+        raise ValueError("slot_append: value rows do not fit the table")
+    _lib.check_mixers(_lib.mixers().gbxm_slot_append(k_rows.data_ptr(), k_rows.stride(0), cache.k_width, v_rows.data_ptr() if two else None,
+                                                    v_rows.stride(0) if two else 0, cache.v_width, cache.keys.data_ptr(),
+                                                    cache.values.data_ptr() if two else None, batch.seq.data_ptr(), batch.tok.data_ptr(), batch.total,
+                                                    cache.keep, cache.ring, act, _stream(k_rows.device)))
+
+
+def sink_attention(q: torch.Tensor, k_new: torch.Tensor, v_new: torch.Tensor, cache, batch, scale: float, window: Optional[int], keep: int,
+                   sink: Optional[torch.Tensor], gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Context rows [T, H * dv]; q [T, H, dk], k_new [T, G, dk], v_new [T, G, dv] views with unit channel stride, gate [T, H] or None;
+    ``cache`` (models/cache.py:SlotKVCache, or None for a step without history) holds the positions before the step."""
+    act = _act(q, "q")
+    t, heads, dk = q.shape
+    groups, dv = v_new.shape[1], v_new.shape[2]
+    if t != batch.total or k_new.shape != (t, groups, dk) or v_new.shape[0] != t or any(x.stride(2) != 1 or x.dtype != q.dtype for x in (q, k_new, v_new)):
+        raise ValueError("sink_attention: q / k / v do not fit the step")
+    if sink is not None and sink.numel() != heads:
+        raise ValueError("sink_attention: one sink per head")
+    if gate is not None and (gate.shape != (t, heads) or gate.stride(1) != 1 or gate.dtype != q.dtype):
+        raise ValueError("sink_attention: gate [T, H] in the activation dtype")
+    a = _lib.SinkAttnArgs()
+    a.q, a.q_row, a.q_head = q.data_ptr(), q.stride(0), q.stride(1)
+    a.k_new, a.k_row, a.k_head = k_new.data_ptr(), k_new.stride(0), k_new.stride(1)
+    a.v_new, a.v_row, a.v_head = v_new.data_ptr(), v_new.stride(0), v_new.stride(1)
+    longest = max(p + n for p, n in zip(batch.pos0, batch.n_new))
+    if cache is not None and cache.keys is not None:
+        kc, vc = cache.keys, cache.values
+        if kc.dtype != q.dtype or kc.shape[0] <= max(batch.slot) or kc.shape[2] < groups * dk or vc.shape[2] < groups * dv:
+            raise ValueError("sink_attention: the table does not fit the step")
+        if cache.window is None and cache.ring < longest:
+            raise ValueError("sink_attention: the table is shorter than the step's longest sequence")
+        a.kcache, a.kc_slot, a.kc_row, a.kc_head = kc.data_ptr(), kc.stride(0), kc.stride(1), dk
+        a.vcache, a.vc_slot, a.vc_row, a.vc_head = vc.data_ptr(), vc.stride(0), vc.stride(1), dv
+        a.keep, a.ring = cache.keep, cache.ring
+    else:
+        if any(batch.pos0):
+            raise ValueError("sink_attention: a step with history needs its table")
+        a.keep, a.ring = (keep, window) if window is not None else (0, 1)
+    if window is not None and (a.keep != keep or a.ring < window):
+        raise ValueError("sink_attention: the table's kept rows / ring do not fit the mask")
+    out = torch.empty((t, heads * dv), dtype=q.dtype, device=q.device)
+    a.seq, a.tok = batch.seq.data_ptr(), batch.tok.data_ptr()
+    a.tiles = batch.tiles.data_ptr() if batch.tiles is not None and batch.tiles.numel() else None
+    a.out = out.data_ptr()
+    a.sink = _f32(sink, "sink").data_ptr() if sink is not None else None
+    if gate is not None:
+        a.gate, a.gate_row = gate.data_ptr(), gate.stride(0)
+    a.T, a.B, a.n_tiles, a.q_tile = t, len(batch.slot), 0 if batch.tiles is None else batch.tiles.shape[0], batch.q_tile
+    a.H, a.G, a.dk, a.dv = heads, groups, dk, dv
+    a.window, a.scale = (0 if window is None else int(window)), float(scale)
+    a.decode_only, a.act = int(batch.decode_only), act
+    partial = None
+    if t * groups < 256 and t <= 64:                            # few rows: room for key-split partial sums
+        # keys of the longest row; launches that are being captured are replayed for longer sequences: size for the table then
+        keys = longest if window is None else min(window + keep, longest)
+        if torch.cuda.is_current_stream_capturing() and cache is not None:
+            keys = cache.rows
+        splits = min(64, (keys + 127) // 128)
+        if splits > 1:
+            partial = torch.empty((splits, t, heads, dv + 2), dtype=torch.float32, device=q.device)
+            a.partial, a.partial_splits = partial.data_ptr(), splits
+    _lib.check_mixers(_lib.mixers().gbxm_sink_attention(ctypes.byref(a), _stream(q.device)))
+    return out

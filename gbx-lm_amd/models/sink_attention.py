@@ -234,7 +234,8 @@ class LatentAttention(nn.Module):
         latent = y[:, self.nq:self.nq + self.nl]                                   # c | rotated key part: the cached row
         gate = y[:, self.nq + self.nl:]
         cache.reserve(max(p + n for p, n in zip(batch.pos0, batch.n_new)), y.dtype, y.device)
-        if not any(batch.pos0):
+        if not any(batch.pos0) and not batch.decode_only:           # (one-token steps always take the form below: a captured step
+                                                                    # is replayed at later positions)
             kv = F.linear(latent[:, :rank], self.up.weight)
             keys = kv[:, :self.nq].view(t, hd, self.dk)
             keys[:, :, d:] = latent[:, None, rank:]

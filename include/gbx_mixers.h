@@ -22,7 +22,7 @@ extern "C" {
 int gbxm_version(void);
 const char* gbxm_last_error(void);
 
-/* x[t] = table[token[t]] * scale (fp32 stream) and its image h in the activation dtype (h may be null when act is fp32). */
+/* x[t] = table[token[t]] * scale (fp32 stream) and its image h in the activation dtype (h may be null: no image is written). */
 int gbxm_embed_scaled(const void* table, const int64_t* tokens, float* x, void* h, int64_t T, int32_t width, float scale,
                       int32_t act, void* stream);
 /* In place: rows[t][0:n0] and rows[t][n0:n0+n1] each RMS-normalised over the whole segment (fp32 statistics), times w0 / w1. */
@@ -73,6 +73,61 @@ int gbxm_window_attention_tiled(int32_t dk, int32_t dv, int32_t act, int32_t dec
 /* Append the step's k / v rows to the rings (only the last `window` rows of a sequence are written). */
 int gbxm_window_append(const void* qkv, int64_t row_stride, int32_t nq, int32_t nk, int32_t nv, void* kcache, void* vcache,
                        const int32_t* seq, const int32_t* tok, int64_t T, int32_t window, int32_t act, void* stream);
+
+/* ---- softmax attention with a sink, rotations, parallel-layer stream update (gbx-lm_amd/models/sink_attention.py) ---- */
+
+/* x[i] += a[i] (+ b[i]) in fp32 over n elements; a, b in the activation dtype (b may be null). */
+int gbxm_stream_add(float* x, const void* a, const void* b, int64_t n, int32_t act, void* stream);
+/* In place on n elements, fp32 arithmetic: kind 1 = relu(z)^2, 2 = gelu in its tanh form. */
+#define GBXM_ACT_RELU2 1
+#define GBXM_ACT_GELU_TANH 2
+int gbxm_activate(void* z, int64_t n, int32_t kind, int32_t act, void* stream);
+
+/* A run of `heads` heads of `head_dim` channels at `offset` of every row.  Channels [rot_offset, rot_offset + rot_dims) of each head
+ * turn by sign * position * freq[i] (pairs i, i + rot_dims/2; or 2i, 2i+1 when interleaved), cos and sin times mult; then the head
+ * is scaled to unit root mean square (norm 1) or RMS-normalised with `weight` [head_dim] (norm 2).  All in fp32, in place. */
+typedef struct {
+  int32_t offset, heads, head_dim, rot_offset, rot_dims, interleaved, norm;
+  float mult, sign;
+  const float* freq;            /* [rot_dims / 2] */
+  const float* weight;          /* [head_dim] for norm 2 */
+} gbxm_head_segment;
+#define GBXM_MAX_SEGMENTS 4
+int gbxm_rotate_norm_heads(void* rows, int64_t T, int64_t row_stride, const int32_t* positions, int64_t pos_stride,
+                           const gbxm_head_segment* segs, int32_t n_segs, float eps, int32_t act, void* stream);
+
+/* Slot tables [slots][keep + ring][width]: position p of a sequence lives in row p (p < keep) or keep + (p - keep) % ring.
+ * Appends the step's rows (key rows, and value rows unless v is null); of two rows of a step that share a place the later stays. */
+int gbxm_slot_append(const void* k, int64_t k_stride, int32_t k_width, const void* v, int64_t v_stride, int32_t v_width, void* kcache,
+                     void* vcache, const int32_t* seq, const int32_t* tok, int64_t T, int32_t keep, int32_t ring, int32_t act, void* stream);
+
+/* out[t][h] = gate * sum_j p_j v_j,  p_j = exp(s_j) / (exp(sink_h) + sum_j exp(s_j)),  s_j = scale <q[t][h], k_j> over the keys
+ * j <= i of the row's sequence with i - j < window or j < keep.  Keys before the step's first row come from the slot tables, the
+ * step's own from k_new / v_new.  Strides in elements; the channel stride is 1 everywhere. */
+typedef struct {
+  const void* q;      int64_t q_row, q_head;          /* [T][H] x dk */
+  const void* k_new;  int64_t k_row, k_head;          /* [T][G] x dk */
+  const void* v_new;  int64_t v_row, v_head;          /* [T][G] x dv */
+  const void* kcache; int64_t kc_slot, kc_row, kc_head;   /* null when no sequence of the step has history */
+  const void* vcache; int64_t vc_slot, vc_row, vc_head;
+  const int32_t* seq;           /* [B][4] */
+  const int32_t* tok;           /* [T][2] */
+  const int32_t* tiles;         /* [n_tiles][2] (prompt kernel) */
+  void* out;                    /* [T][H*dv] */
+  const float* sink;            /* [H], or null: plain softmax */
+  const void* gate;  int64_t gate_row;                /* [T][H] activation dtype, or null: out *= sigmoid(gate) */
+  int64_t T;
+  int32_t B, n_tiles, q_tile;
+  int32_t H, G, dk, dv;
+  int32_t window;               /* <= 0: every earlier key is seen */
+  int32_t keep, ring;
+  float scale;
+  int32_t decode_only, act;
+  void* partial;                /* optional fp32 [partial_splits][T][H][dv + 2] */
+  int32_t partial_splits;
+} gbxm_sink_attn_args;
+int gbxm_sink_attention(const gbxm_sink_attn_args* a, void* stream);
+int gbxm_sink_attention_tiled(int32_t dk, int32_t dv, int32_t act, int32_t decode_only);
 
 #ifdef __cplusplus
 }
