@@ -555,11 +555,83 @@ def revitar_bench(args):
     print(json.dumps({"metric": "revitar_throughput", "unit": "tokens/s", "dtype": "bf16", "data": "synthetic", "sizes": out}))
 
 
+RADENEX_SIZES = {
+    # name: Radenex geometry (latent attention and windowed attention layers alternate; the span runs twice) and, from it, the Revitar
+    # (the closest existing model: the other dense bf16 decoder over ragged steps, windowed attention) of equal width / heads / window
+    "small": dict(width=1024, latent=dict(heads=8, dim=64, rot_dim=32, vdim=64, kv_rank=256),
+                  attention=dict(heads=16, kv_heads=4, dim=64, vdim=64, window=1024, keep_first=4), ff=4096, pattern="la", loop=(0, 2, 2)),
+    "lite-like": dict(width=2048, latent=dict(heads=16, dim=128, rot_dim=64, vdim=128, kv_rank=512),
+                      attention=dict(heads=16, kv_heads=4, dim=128, vdim=128, window=4096, keep_first=4), ff=8192, pattern="la", loop=(0, 2, 2)),
+    "wide": dict(width=4096, latent=dict(heads=32, dim=128, rot_dim=64, vdim=128, kv_rank=512),
+                 attention=dict(heads=32, kv_heads=8, dim=128, vdim=128, window=2048, keep_first=4), ff=8192, pattern="la", loop=None),
+}
+
+
+def radenex_bench(args):
+    """``--design radenex``: prefill and decode throughput of Radenex at layer sizes of real models (random weights, bf16), beside
+    Revitar with the attention layer's geometry in every layer and one always-chosen expert of the same feed-forward width (equal
+    layer runs).  One JSON line; the default workload of this file is untouched."""
+    from gbx_lm_amd import synthetic as S
+    from gbx_lm_amd.batching import BatchScheduler
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+
+    def clock(fn, reps):
+        fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / reps
+
+    def legs(model, vocab, window, tag, res):
+        toks = lambda n, o=0: [(o + i * 7919) % vocab for i in range(n)]
+        for T in (512, 4096):
+            def prefill():
+                eng = BatchScheduler(model)
+                eng.step([("p", toks(T))])
+            res[f"{tag}prefill_T{T}_tok_s"] = round(T / clock(prefill, 3) * 1e3)
+        for B, ctx in ((1, 2048), (32, 256)):
+            eng = BatchScheduler(model)
+            eng.step([(i, toks(ctx, i)) for i in range(B)])
+            state = {"t": 0}
+            def decode():
+                state["t"] += 1
+                eng.step([(i, [(state["t"] * 31 + i) % vocab]) for i in range(B)])
+            res[f"{tag}decode_B{B}_ctx{ctx}_tok_s"] = round(B / clock(decode, 64) * 1e3)
+            del eng
+        print(tag or "radenex", res, file=sys.stderr, flush=True)
+
+    out = {}
+    for name in args.sizes.split(","):
+        g = RADENEX_SIZES[name]
+        res = {"geometry": g}
+        cfg = S.radenex_config(**g)
+        model = S.build_radenex(cfg, device=dev, seed=0)
+        res["layer_runs"] = len(model.layers)
+        legs(model, cfg["vocab"], g["attention"]["window"], "", res)
+        runs = len(model.layers)
+        del model
+        torch.cuda.empty_cache()
+        a = g["attention"]
+        rm = S.build_revitar(S.revitar_config(width=g["width"], heads=a["heads"], kv_heads=a["kv_heads"], dim=a["dim"], vdim=a["vdim"],
+                                              window=a["window"], experts=1, top=1, ff=g["ff"], n_layers=runs, vocab=cfg["vocab"]), device=dev, seed=0)
+        legs(rm, cfg["vocab"], a["window"], "revitar_", res)
+        del rm
+        torch.cuda.empty_cache()
+        out[name] = res
+    print(json.dumps({"metric": "radenex_throughput", "unit": "tokens/s", "dtype": "bf16", "data": "synthetic", "sizes": out}))
+
+
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--design", default=None, choices=["revitar"], help="side benchmark of one model design beside the closest existing "
+    ap.add_argument("--design", default=None, choices=["revitar", "radenex"], help="side benchmark of one model design beside the closest existing "
                     "family at equal size (own JSON line; the default workload and its output are unchanged)")
-    ap.add_argument("--sizes", default="small,a3b-like", help="--design revitar: comma-separated names of REVITAR_SIZES")
+    ap.add_argument("--sizes", default=None, help="--design: comma-separated names of REVITAR_SIZES (default small,a3b-like) / RADENEX_SIZES "
+                    "(default small,lite-like)")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=512, help="timed decode steps (default: > 0.5 s of GPU time, so that a coarse GPU-busy sampler sees the run)")
     ap.add_argument("--warmup", type=int, default=8)
@@ -575,10 +647,11 @@ def main():
     ap.add_argument("--dry-run", action="store_true", help="CPU / gloo rehearsal of the multi-rank control flow")
     args = ap.parse_args()
 
-    if args.design == "revitar":
+    if args.design is not None:
         if not torch.cuda.is_available():
             raise SystemExit("bench.py needs an MI355X")
-        return revitar_bench(args)
+        args.sizes = args.sizes or {"revitar": "small,a3b-like", "radenex": "small,lite-like"}[args.design]
+        return revitar_bench(args) if args.design == "revitar" else radenex_bench(args)
     if args.gpus > 1 and "WORLD_SIZE" not in os.environ:
         spawn_ranks(args.gpus)                                     # never returns; nothing has touched the GPU yet
     world = int(os.environ.get("WORLD_SIZE", "1"))

@@ -291,3 +291,75 @@ def build_revitar(config: Dict, device="cpu", seed: int = 0, act_dtype=torch.bfl
             m._buffers[attr] = torch.ones(tuple(b.shape), dtype=torch.float32, device=device)
     model.eval()
     return model
+
+
+# ------------------------------------------------------------------------------------------------ Radenex (dense, parallel layers)
+def radenex_config(width: int, latent: Dict, attention: Dict, ff: int, pattern: str = "la", loop=None, vocab: int = 32000) -> Dict:
+    """config.json of a Radenex model: ``pattern`` names the layers in order ('l' latent attention, 'a' windowed attention), every
+    layer with a dense feed-forward of ``ff`` channels; ``loop`` = (start, stop, times) or None.
+    ``latent``: heads, dim, rot_dim, vdim, kv_rank; ``attention``: heads, kv_heads, dim, vdim, window, keep_first."""
+    lat = {"type": "latent_attention",
+           "mixer": {"heads": latent["heads"], "dim": latent["dim"], "rot_dim": latent["rot_dim"], "vdim": latent["vdim"],
+                     "kv_rank": latent["kv_rank"], "scale": (latent["dim"] + latent["rot_dim"]) ** -0.5,
+                     "rot": {"base": 10000.0, "dims": latent["rot_dim"],
+                             "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}},
+           "mlp": {"kind": "dense", "ff": ff}}
+    att = {"type": "attention",
+           "mixer": {"heads": attention["heads"], "kv_heads": attention["kv_heads"], "dim": attention["dim"], "vdim": attention["vdim"],
+                     "mask": {"size": attention["window"], "keep_first": attention.get("keep_first", 0)}, "scale": attention["dim"] ** -0.5,
+                     "rot": {"base": 10000.0, "dims": attention.get("rot_dims", attention["dim"]), "scaling": {"factor": 2.0}}},
+           "mlp": {"kind": "dense", "ff": ff}}
+    cfg = {"architecture": "Radenex", "vocab": vocab, "width": width, "norm": {"eps": 1e-6},
+           "layers": [json.loads(json.dumps(lat if c == "l" else att)) for c in pattern]}
+    if loop:
+        cfg["loop"] = {"start": loop[0], "stop": loop[1], "times": loop[2]}
+    return cfg
+
+
+def build_radenex(config: Dict, device="cpu", seed: int = 0, act_dtype=torch.bfloat16):
+    """Random-init Radenex with real shapes, generated directly on ``device`` (no files)."""
+    from .models import radenex
+    from .models.sink_attention import LatentAttention
+    device = torch.device(device)
+    args = radenex.ModelArgs.from_dict(config)
+    tables = {}
+    model = radenex.Model(args)                   # on the host first: the frequency tables are computed in the constructors
+    for name, b in model.named_buffers():
+        if name.endswith("freq"):
+            tables[name] = b.clone()
+    with torch.device("meta"):
+        model = radenex.Model(args)
+    model = model.to_empty(device=device)
+    gen = torch.Generator(device=device)
+    gen.manual_seed(seed)
+
+    def rnd(shape, std, dtype):
+        return (torch.randn(tuple(shape), device=device, generator=gen) * std).to(dtype)
+
+    mods = dict(model.named_modules())
+    for name, p in list(model.named_parameters()):
+        mod, _, attr = name.rpartition(".")
+        std = 1.0 if "embed_tokens" in name else p.shape[-1] ** -0.5
+        mods[mod]._parameters[attr] = torch.nn.Parameter(rnd(p.shape, std, act_dtype), requires_grad=False)
+    for name, b in list(model.named_buffers()):
+        mod, _, attr = name.rpartition(".")
+        m = mods[mod]
+        if name in tables:
+            m._buffers[attr] = tables[name].to(device)
+        elif attr == "sink":
+            m._buffers[attr] = (torch.rand(tuple(b.shape), device=device, generator=gen) if isinstance(m, LatentAttention)
+                                else torch.zeros(tuple(b.shape), device=device))
+        elif attr in ("uk_heads", "uv_heads_t"):
+            pass                                   # cut from the key / value product below
+        else:                                      # norm weights
+            m._buffers[attr] = torch.ones(tuple(b.shape), dtype=torch.float32, device=device)
+    for m in model.modules():                      # the per-head images are views of the same numbers as the whole-prompt product
+        if isinstance(m, LatentAttention):
+            h, d, r, dv, rank = m.heads, m.dim, m.rot_dim, m.vdim, m.kv_rank
+            up = m.up.weight.data
+            keys = up[:h * (d + r)].view(h, d + r, rank)
+            keys[:, d:] = 0
+            m._buffers["uk_heads"] = keys[:, :d].contiguous()
+            m._buffers["uv_heads_t"] = up[h * (d + r):].view(h, dv, rank).transpose(1, 2).contiguous()
+    model.eval()
+    return model
