@@ -365,7 +365,14 @@ bool act_ok(int act) { return act == GBXM_BF16 || act == GBXM_F32; }
 }  // namespace
 
 int launch_sink_tiles(const gbxm_sink_attn_args& a, hipStream_t s);     // mixers_sink_mfma.hip; GBXM_ERR_UNSUPPORTED: not its shape
+int launch_sink_group(const gbxm_sink_attn_args& a, hipStream_t s);     // the same for steps of single rows
 bool sink_tiles_shape(int dk, int dv);
+
+int launch_sink_reduce(const gbxm_sink_attn_args& a, int splits, hipStream_t s) {
+  sink_reduce_kernel<bf16_t, true><<<dim3(a.T, a.H), 128, 0, s>>>(static_cast<const float*>(a.partial), static_cast<bf16_t*>(a.out), a.sink,
+                                                                  static_cast<const bf16_t*>(a.gate), a.gate_row, a.T, a.H, a.dv, splits);
+  return after_launch("sink_attention (join of key splits)");
+}
 
 }  // namespace gbxm
 
@@ -430,7 +437,7 @@ int gbxm_slot_append(const void* k, int64_t k_stride, int32_t k_width, const voi
 }
 
 int gbxm_sink_attention_tiled(int32_t dk, int32_t dv, int32_t act, int32_t decode_only) {
-  return act == GBXM_BF16 && !decode_only && sink_tiles_shape(dk, dv);
+  return act == GBXM_BF16 && sink_tiles_shape(dk, dv);          // (steps of single rows: the grouped form of the same products)
 }
 
 int gbxm_sink_attention(const gbxm_sink_attn_args* a, void* stream) {
@@ -444,6 +451,10 @@ int gbxm_sink_attention(const gbxm_sink_attn_args* a, void* stream) {
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (!a->decode_only && a->act == GBXM_BF16 && a->tiles && a->n_tiles > 0) {
     const int rc = launch_sink_tiles(*a, s);
+    if (rc != GBXM_ERR_UNSUPPORTED) return rc;
+  }
+  if (a->decode_only && a->act == GBXM_BF16 && a->H <= 65535) {
+    const int rc = launch_sink_group(*a, s);
     if (rc != GBXM_ERR_UNSUPPORTED) return rc;
   }
   SinkGeo g{a->H, a->G, a->dk, a->dv, a->window, a->keep, a->ring, a->scale, a->q_row, a->q_head, a->k_row, a->k_head, a->v_row, a->v_head,

@@ -10,9 +10,13 @@
 // for the value product; the denominator sums them in fp32.
 //
 // Head sizes are run-time numbers (multiples of 8) inside a compiled capacity <DK, DV>: channels beyond them are staged as zeros.
+#include <algorithm>
 #include "mixers_mfma.h"
 
 namespace gbxm {
+
+int launch_sink_reduce(const gbxm_sink_attn_args& a, int splits, hipStream_t s);      // mixers_sink.hip
+
 namespace {
 
 struct SinkTileArgs {
@@ -43,7 +47,8 @@ __global__ __launch_bounds__(256) void sink_tile_kernel(const SinkTileArgs a) {
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 31, hb = lane >> 5;
-  const int b = a.tiles[2 * blockIdx.x], tq = a.tiles[2 * blockIdx.x + 1];
+  const int tile = gridDim.x - 1 - blockIdx.x;               // a sequence's late tiles see the most keys: they are scheduled first
+  const int b = a.tiles[2 * tile], tq = a.tiles[2 * tile + 1];
   const int head = blockIdx.y, kvh = head / (a.H / a.G);
   const int slot = a.seq[4 * b], pos0 = a.seq[4 * b + 1], n = a.seq[4 * b + 2], row0 = a.seq[4 * b + 3];
   const int W = a.window;
@@ -74,9 +79,10 @@ __global__ __launch_bounds__(256) void sink_tile_kernel(const SinkTileArgs a) {
   const bool wave_live = wave * 32 < qn;
   const int wq0 = qfirst + wave * 32, wq1 = min(wq0 + 31, jlast);      // positions of this wave's queries
 
-  float m = a.sink ? a.sink[head] : -INFINITY;
+  constexpr float LOG2E = 1.4426950408889634f;
+  const float scale2 = a.scale * LOG2E;
+  float m = a.sink ? a.sink[head] * LOG2E : -INFINITY;
   float l = (a.sink && hb == 0) ? 1.f : 0.f;                            // the sink counts once per query
-  const float scale = a.scale;
   const unsigned char* vbase = vl + (4 * hb + ((lane >> 2) & 3)) * VROW + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
   const unsigned char* kbase = kl + r * KROW + hb * 16;
 
@@ -127,29 +133,40 @@ __global__ __launch_bounds__(256) void sink_tile_kernel(const SinkTileArgs a) {
     f32x16 st = f32x16{0};
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) st = mfma_bf16(*reinterpret_cast<const u32x4*>(kbase + ks * 32), qf[ks], st);
+    // scores in units of ln 2 (the exponentials below are base 2).  Inside the mask -- every key of the tile before every query of the
+    // wave, inside every window -- nothing is tested per score.
+    const bool inside = it + KT <= total && jmax <= wq0 && (W <= 0 || wq1 - jmin < W || jmax < a.keep);
     float s[16];
     float mx = -INFINITY;
+    if (inside) {
 #pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      const int iv = it + 8 * (e >> 2) + 4 * hb + (e & 3);
-      const int j = pos_of(iv);
-      const bool seen = qvalid && iv < total && j <= qpos && (W <= 0 || qpos - j < W || j < a.keep);
-      s[e] = seen ? st[e] * scale : -INFINITY;
-      mx = fmaxf(mx, s[e]);
+      for (int e = 0; e < 16; ++e) { s[e] = st[e] * scale2; mx = fmaxf(mx, s[e]); }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int iv = it + 8 * (e >> 2) + 4 * hb + (e & 3);
+        const int j = pos_of(iv);
+        const bool seen = qvalid && iv < total && j <= qpos && (W <= 0 || qpos - j < W || j < a.keep);
+        s[e] = seen ? st[e] * scale2 : -INFINITY;
+        mx = fmaxf(mx, s[e]);
+      }
     }
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));                   // the other half of the query's scores
     const float m_new = fmaxf(m, mx);
-    const float m_ref = m_new == -INFINITY ? 0.f : m_new;     // nothing seen yet and no sink: every weight below is exp(-inf) = 0
-    const float alpha = __expf(m - m_ref);
+    const float m_ref = m_new == -INFINITY ? 0.f : m_new;     // nothing seen yet and no sink: every weight below is 2^-inf = 0
+    const float alpha = __builtin_amdgcn_exp2f(m - m_ref);
+    const bool moved = m_new != m;
     m = m_new;
     float ps = 0.f;
 #pragma unroll
-    for (int e = 0; e < 16; ++e) { s[e] = __expf(s[e] - m_ref); ps += s[e]; }
+    for (int e = 0; e < 16; ++e) { s[e] = __builtin_amdgcn_exp2f(s[e] - m_ref); ps += s[e]; }
     l = l * alpha + ps;
+    if (__any(moved)) {                                       // wave-uniform: the maximum of no query of the wave has moved -> alpha is 1
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
+      for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) o[dt][e] *= alpha;
+        for (int e = 0; e < 16; ++e) o[dt][e] *= alpha;
+    }
     u32x4 gf[2];
 #pragma unroll
     for (int tt = 0; tt < 2; ++tt)
@@ -182,6 +199,172 @@ __global__ __launch_bounds__(256) void sink_tile_kernel(const SinkTileArgs a) {
   }
 }
 
+// Steps of single rows (decoding): the query heads that share a key/value head are the 32 "query rows" of the same two products,
+// all at one position, so a key tile staged once serves every head of the group.  One workgroup = one (row, kv head, 32 heads of
+// its group, share of the key tiles); every wave forms all scores of a tile (the weights must be the same in all of them) and
+// owns every fourth 32-channel block of the value product.  No mask besides the end of the key run.  With key splits a workgroup
+// leaves (sum, maximum, denominator) per head for sink_reduce_kernel, else it finishes the row itself.
+// ALIAS: the values are the first dv channels of the key rows (one staged tile serves both products).
+template <int DK, int DV, bool ALIAS>
+__global__ __launch_bounds__(256) void sink_group_kernel(const SinkTileArgs a, const int* __restrict__ tok, int splits, float* __restrict__ partial) {
+  constexpr int KT = 32;
+  constexpr int KROW = DK * 2 + 16;
+  constexpr int VROW = ALIAS ? KROW : DV * 2 + 64;
+  constexpr int KS = DK / 16, DT = DV / 32, DTW = (DT + 3) / 4;
+  __shared__ __attribute__((aligned(16))) unsigned char lds[KT * KROW + (ALIAS ? 0 : KT * VROW)];
+  unsigned char* kl = lds;
+  unsigned char* vl = ALIAS ? lds : lds + KT * KROW;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 31, hb = lane >> 5;
+  const int64_t t = blockIdx.x;
+  const int R = a.H / a.G, chunks = (R + 31) / 32;
+  const int kvh = blockIdx.y / chunks, hloc = (blockIdx.y % chunks) * 32 + r;
+  const bool hvalid = hloc < R;
+  const int head = kvh * R + min(hloc, R - 1);
+  const int b = tok[2 * t], pos = tok[2 * t + 1];
+  const int slot = a.seq[4 * b], pos0 = a.seq[4 * b + 1], row0 = a.seq[4 * b + 3];
+  const int W = a.window;
+
+  u32x4 qf[KS];
+  {
+    const bf16_t* qp = a.q + t * a.q_row + head * a.q_head;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int c = ks * 16 + hb * 8;
+      qf[ks] = c < a.dk ? *reinterpret_cast<const u32x4*>(qp + c) : u32x4{0, 0, 0, 0};
+    }
+  }
+  f32x16 o[DTW];
+#pragma unroll
+  for (int i = 0; i < DTW; ++i) o[i] = f32x16{0};
+
+  const int lo = W > 0 ? max(0, pos - W + 1) : 0;
+  const int na = min(a.keep, lo);
+  const int total = na + (pos - lo + 1);
+  auto pos_of = [&](int iv) { return iv < na ? iv : lo + (iv - na); };
+  auto krow = [&](int j) -> const bf16_t* {
+    if (j < pos0) return a.kc + slot * a.kc_slot + static_cast<int64_t>(j < a.keep ? j : a.keep + (j - a.keep) % a.ring) * a.kc_row + kvh * a.kc_head;
+    return a.kn + static_cast<int64_t>(row0 + (j - pos0)) * a.k_row + kvh * a.k_head;
+  };
+  auto vrow = [&](int j) -> const bf16_t* {
+    if (j < pos0) return a.vc + slot * a.vc_slot + static_cast<int64_t>(j < a.keep ? j : a.keep + (j - a.keep) % a.ring) * a.vc_row + kvh * a.vc_head;
+    return a.vn + static_cast<int64_t>(row0 + (j - pos0)) * a.v_row + kvh * a.v_head;
+  };
+
+  constexpr float LOG2E = 1.4426950408889634f;
+  const float scale2 = a.scale * LOG2E;
+  const bool own_sink = a.sink && splits == 1;                          // split key tiles: the sink joins in the reduce
+  float m = own_sink ? a.sink[head] * LOG2E : -INFINITY;
+  float l = (own_sink && hb == 0) ? 1.f : 0.f;
+  const unsigned char* vbase = vl + (4 * hb + ((lane >> 2) & 3)) * VROW + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
+  const unsigned char* kbase = kl + r * KROW + hb * 16;
+
+  for (int it = static_cast<int>(blockIdx.z) * KT; it < total; it += KT * splits) {
+    __syncthreads();                                          // the previous tile has been consumed
+    for (int p = tid; p < KT * (DK / 8); p += 256) {
+      const int row = p / (DK / 8), c = p % (DK / 8), iv = it + row;
+      u32x4 v = u32x4{0, 0, 0, 0};
+      if (iv < total && c * 8 < a.dk) v = *reinterpret_cast<const u32x4*>(krow(pos_of(iv)) + c * 8);
+      *reinterpret_cast<u32x4*>(kl + row * KROW + c * 16) = v;
+    }
+    if constexpr (!ALIAS) {
+      for (int p = tid; p < KT * (DV / 8); p += 256) {
+        const int row = p / (DV / 8), c = p % (DV / 8), iv = it + row;
+        u32x4 v = u32x4{0, 0, 0, 0};
+        if (iv < total && c * 8 < a.dv) v = *reinterpret_cast<const u32x4*>(vrow(pos_of(iv)) + c * 8);
+        *reinterpret_cast<u32x4*>(vl + row * VROW + c * 16) = v;
+      }
+    }
+    __syncthreads();
+    f32x16 st = f32x16{0};
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) st = mfma_bf16(*reinterpret_cast<const u32x4*>(kbase + ks * 32), qf[ks], st);
+    float s[16];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const int iv = it + 8 * (e >> 2) + 4 * hb + (e & 3);
+      s[e] = iv < total ? st[e] * scale2 : -INFINITY;
+      mx = fmaxf(mx, s[e]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));                   // finite: a tile holds at least one key
+    const float m_new = fmaxf(m, mx);
+    const float alpha = __builtin_amdgcn_exp2f(m - m_new);
+    m = m_new;
+    float ps = 0.f;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) { s[e] = __builtin_amdgcn_exp2f(s[e] - m_new); ps += s[e]; }
+    l = l * alpha + ps;
+    u32x4 gf[2];
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt)
+      gf[tt] = u32x4{pack2(s[8 * tt], s[8 * tt + 1]), pack2(s[8 * tt + 2], s[8 * tt + 3]), pack2(s[8 * tt + 4], s[8 * tt + 5]),
+                     pack2(s[8 * tt + 6], s[8 * tt + 7])};
+#pragma unroll
+    for (int i = 0; i < DTW; ++i) {
+      const int dt = wave + 4 * i;                            // wave-uniform
+      if (dt < DT) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) o[i][e] *= alpha;
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt) {
+          const u32x2 v0 = lds_read_tr(vbase + (16 * tt) * VROW + dt * 64);
+          const u32x2 v1 = lds_read_tr(vbase + (16 * tt + 8) * VROW + dt * 64);
+          o[i] = mfma_bf16(u32x4{v0.x, v0.y, v1.x, v1.y}, gf[tt], o[i]);
+        }
+      }
+    }
+  }
+
+  l += __shfl_xor(l, 32, 64);
+  if (!hvalid) return;
+  if (splits > 1) {
+    float* prow = partial + ((static_cast<int64_t>(blockIdx.z) * gridDim.x + t) * a.H + head) * (a.dv + 2);
+#pragma unroll
+    for (int i = 0; i < DTW; ++i) {
+      const int dt = wave + 4 * i;
+      if (dt < DT)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int d = dt * 32 + 8 * (e >> 2) + 4 * hb + (e & 3);
+          if (d < a.dv) prow[d] = o[i][e];
+        }
+    }
+    if (wave == 0 && hb == 0) { prow[a.dv] = m / LOG2E; prow[a.dv + 1] = l; }
+    return;
+  }
+  float f = 1.f / l;
+  if (a.gate) f *= sigmoid_<true>(to_f32(a.gate[t * a.gate_row + head]));
+  bf16_t* op = a.out + t * (static_cast<int64_t>(a.H) * a.dv) + head * a.dv;
+#pragma unroll
+  for (int i = 0; i < DTW; ++i) {
+    const int dt = wave + 4 * i;
+    if (dt < DT)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const int d = dt * 32 + 8 * q4 + 4 * hb;
+        if (d < a.dv)
+          *reinterpret_cast<u32x2*>(op + d) = u32x2{pack2(o[i][4 * q4] * f, o[i][4 * q4 + 1] * f), pack2(o[i][4 * q4 + 2] * f, o[i][4 * q4 + 3] * f)};
+      }
+  }
+}
+
+template <int DK, int DV, bool ALIAS>
+int launch_group(const SinkTileArgs& t, const gbxm_sink_attn_args& a, hipStream_t s) {
+  const int R = a.H / a.G, chunks = (R + 31) / 32;
+  int splits = 1;
+  const int64_t groups = a.T * a.G * chunks;
+  if (a.partial && a.partial_splits > 1 && groups < 256) {
+    splits = static_cast<int>(std::min<int64_t>(std::min<int64_t>(512 / groups, 64), a.partial_splits));
+    if (splits < 2) splits = 1;
+  }
+  sink_group_kernel<DK, DV, ALIAS><<<dim3(a.T, a.G * chunks, splits), 256, 0, s>>>(t, a.tok, splits, static_cast<float*>(a.partial));
+  const int rc = after_launch("sink_attention (grouped rows)");
+  if (rc != GBXM_OK || splits == 1) return rc;
+  return launch_sink_reduce(a, splits, s);
+}
+
 template <int DK, int DV>
 int launch(const SinkTileArgs& t, int n_tiles, hipStream_t s) {
   sink_tile_kernel<DK, DV><<<dim3(n_tiles, t.H), 256, 0, s>>>(t);
@@ -199,19 +382,58 @@ bool sink_tiles_shape(int dk, int dv) {
   return false;
 }
 
+static bool aligned16(const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; }
+
+static bool tile_operands(const gbxm_sink_attn_args& a) {
+  if ((a.q_row | a.q_head | a.k_row | a.k_head | a.v_row | a.v_head) % 8 || !aligned16(a.q) || !aligned16(a.k_new) || !aligned16(a.v_new) ||
+      !aligned16(a.out))
+    return false;
+  if (a.kcache && ((a.kc_slot | a.kc_row | a.kc_head | a.vc_slot | a.vc_row | a.vc_head) % 8 || !aligned16(a.kcache) || !aligned16(a.vcache))) return false;
+  return true;
+}
+
+static SinkTileArgs tile_args(const gbxm_sink_attn_args& a) {
+  return SinkTileArgs{static_cast<const bf16_t*>(a.q), static_cast<const bf16_t*>(a.k_new), static_cast<const bf16_t*>(a.v_new),
+                      static_cast<const bf16_t*>(a.kcache), static_cast<const bf16_t*>(a.vcache), a.seq, a.tiles, static_cast<bf16_t*>(a.out), a.sink,
+                      static_cast<const bf16_t*>(a.gate), a.q_row, a.q_head, a.k_row, a.k_head, a.v_row, a.v_head, a.kc_slot, a.kc_row, a.kc_head,
+                      a.vc_slot, a.vc_row, a.vc_head, a.gate_row, a.q_tile, a.H, a.G, a.dk, a.dv, a.window, a.keep, a.ring, a.scale};
+}
+
 int launch_sink_tiles(const gbxm_sink_attn_args& a, hipStream_t s) {
-  if (!sink_tiles_shape(a.dk, a.dv) || a.q_tile != 128 || a.H > 65535) return GBXM_ERR_UNSUPPORTED;
-  auto al = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
-  if ((a.q_row | a.q_head | a.k_row | a.k_head | a.v_row | a.v_head) % 8 || !al(a.q) || !al(a.k_new) || !al(a.v_new) || !al(a.out))
-    return GBXM_ERR_UNSUPPORTED;
-  if (a.kcache && ((a.kc_slot | a.kc_row | a.kc_head | a.vc_slot | a.vc_row | a.vc_head) % 8 || !al(a.kcache) || !al(a.vcache))) return GBXM_ERR_UNSUPPORTED;
-  SinkTileArgs t{static_cast<const bf16_t*>(a.q), static_cast<const bf16_t*>(a.k_new), static_cast<const bf16_t*>(a.v_new),
-                 static_cast<const bf16_t*>(a.kcache), static_cast<const bf16_t*>(a.vcache), a.seq, a.tiles, static_cast<bf16_t*>(a.out), a.sink,
-                 static_cast<const bf16_t*>(a.gate), a.q_row, a.q_head, a.k_row, a.k_head, a.v_row, a.v_head, a.kc_slot, a.kc_row, a.kc_head,
-                 a.vc_slot, a.vc_row, a.vc_head, a.gate_row, a.q_tile, a.H, a.G, a.dk, a.dv, a.window, a.keep, a.ring, a.scale};
+  if (!sink_tiles_shape(a.dk, a.dv) || a.q_tile != 128 || a.H > 65535 || !tile_operands(a)) return GBXM_ERR_UNSUPPORTED;
+  const SinkTileArgs t = tile_args(a);
 #define GBXM_TILE(DK_, DV_) if (a.dk <= DK_ && a.dv <= DV_) return launch<DK_, DV_>(t, a.n_tiles, s)
   GBXM_TILE(32, 32); GBXM_TILE(64, 64); GBXM_TILE(64, 128); GBXM_TILE(96, 96); GBXM_TILE(128, 128); GBXM_TILE(192, 128); GBXM_TILE(256, 256);
 #undef GBXM_TILE
+  return GBXM_ERR_UNSUPPORTED;
+}
+
+// values that are the leading channels of the key rows (same buffers, same strides): one staged tile serves both products
+static bool values_alias_keys(const gbxm_sink_attn_args& a) {
+  return a.G == 1 && a.dv <= a.dk && a.v_new == a.k_new && a.v_row == a.k_row &&
+         (!a.kcache || (a.vcache == a.kcache && a.vc_slot == a.kc_slot && a.vc_row == a.kc_row));
+}
+
+bool sink_group_shape(int dk, int dv, bool alias) {
+  if (dk % 8 || dv % 8) return false;
+  if (alias) return dk <= 576 && dv <= 512;
+  return sink_tiles_shape(dk, dv);
+}
+
+int launch_sink_group(const gbxm_sink_attn_args& a, hipStream_t s) {
+  const bool alias = values_alias_keys(a);
+  const int chunks = (a.H / a.G + 31) / 32;
+  if (!sink_group_shape(a.dk, a.dv, alias) || a.G * chunks > 65535 || !tile_operands(a)) return GBXM_ERR_UNSUPPORTED;
+  const SinkTileArgs t = tile_args(a);
+  if (alias) {
+#define GBXM_GROUP(DK_, DV_) if (a.dk <= DK_ && a.dv <= DV_) return launch_group<DK_, DV_, true>(t, a, s)
+    GBXM_GROUP(96, 96); GBXM_GROUP(160, 128); GBXM_GROUP(320, 256); GBXM_GROUP(576, 512);
+#undef GBXM_GROUP
+    return GBXM_ERR_UNSUPPORTED;
+  }
+#define GBXM_GROUP(DK_, DV_) if (a.dk <= DK_ && a.dv <= DV_) return launch_group<DK_, DV_, false>(t, a, s)
+  GBXM_GROUP(32, 32); GBXM_GROUP(64, 64); GBXM_GROUP(64, 128); GBXM_GROUP(96, 96); GBXM_GROUP(128, 128); GBXM_GROUP(192, 128); GBXM_GROUP(256, 256);
+#undef GBXM_GROUP
   return GBXM_ERR_UNSUPPORTED;
 }
 

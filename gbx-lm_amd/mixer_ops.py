@@ -257,7 +257,7 @@ def sink_attention(q: torch.Tensor, k_new: torch.Tensor, v_new: torch.Tensor, ca
         keys = longest if window is None else min(window + keep, longest)
         if torch.cuda.is_current_stream_capturing() and cache is not None:
             keys = cache.rows
-        splits = min(64, (keys + 127) // 128)
+        splits = min(64, (keys + 63) // 64)
         if splits > 1:
             partial = torch.empty((splits, t, heads, dv + 2), dtype=torch.float32, device=q.device)
             a.partial, a.partial_splits = partial.data_ptr(), splits

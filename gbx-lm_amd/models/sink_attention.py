@@ -198,7 +198,8 @@ class LatentAttention(nn.Module):
         self.scale, self.eps = float(scale), float(eps)
         self.dk = dim + rot_dim
         self.nq, self.nl = heads * self.dk, kv_rank + rot_dim
-        self.inp = nn.Linear(width, self.nq + self.nl + heads, bias=False)         # q | latent, rotated key part | gate
+        # q | latent, rotated key part | gate, padded with empty rows to a multiple of 8 (rows of the product start 16-byte aligned)
+        self.inp = nn.Linear(width, (self.nq + self.nl + heads + 7) // 8 * 8, bias=False)
         # rows of every head's key product, padded with rot_dim empty rows per head (the shared rotated part is written there), then
         # the value product: one matrix product forms every head's keys and values of a whole prompt
         self.up = nn.Linear(kv_rank, heads * (self.dk + vdim), bias=False)
@@ -219,7 +220,8 @@ class LatentAttention(nn.Module):
         """The module's matrices from the checkpoint's (all [out, in])."""
         h, d, r, dv, rank = self.heads, self.dim, self.rot_dim, self.vdim, self.kv_rank
         uk_pad = torch.cat([uk.view(h, d, rank), torch.zeros((h, r, rank), dtype=uk.dtype)], dim=1).reshape(h * (d + r), rank)
-        return {"inp.weight": torch.cat([q, dkv, g]), "up.weight": torch.cat([uk_pad, uv]),
+        pad = torch.zeros((self.inp.out_features - (self.nq + self.nl + h), q.shape[1]), dtype=q.dtype)
+        return {"inp.weight": torch.cat([q, dkv, g, pad]), "up.weight": torch.cat([uk_pad, uv]),
                 "uk_heads": uk.view(h, d, rank).contiguous(), "uv_heads_t": uv.view(h, dv, rank).transpose(1, 2).contiguous()}
 
     def forward(self, h: torch.Tensor, batch, cache: SlotKVCache) -> torch.Tensor:
@@ -232,7 +234,7 @@ class LatentAttention(nn.Module):
             HeadSegment(self.nq + rank, 1, r, 0, r, self.freq, self.rot_mult)], self.eps)
         q = y[:, :self.nq].view(t, hd, self.dk)
         latent = y[:, self.nq:self.nq + self.nl]                                   # c | rotated key part: the cached row
-        gate = y[:, self.nq + self.nl:]
+        gate = y[:, self.nq + self.nl:self.nq + self.nl + hd]
         cache.reserve(max(p + n for p, n in zip(batch.pos0, batch.n_new)), y.dtype, y.device)
         if not any(batch.pos0) and not batch.decode_only:           # (one-token steps always take the form below: a captured step
                                                                     # is replayed at later positions)

@@ -287,13 +287,15 @@ def test_feed_forward_and_stream_update(device, dtype):
 
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("kind", ["latent", "attention", "latent_odd", "attention_wide"])
+@pytest.mark.parametrize("kind", ["latent", "attention", "latent_odd", "attention_wide", "latent_wide", "latent_many_heads"])
 def test_mixers_alone(device, dtype, kind):
     """One mixer module with random weights: a whole prompt (keys and values formed per head), then token by token and in portions
     (the latent mixer attends over its cached rows directly there)."""
     g = torch.Generator().manual_seed(4)
     W, T, eps = 72, 90, 1e-5
     layer = {"latent": O.latent_layer(4, 16, 8, 24, 32, scaling=YARN), "latent_odd": O.latent_layer(3, 10, 6, 14, 18, base=77.0),
+             "latent_wide": O.latent_layer(16, 64, 32, 64, 256),                          # one latent row of 288 channels for 16 heads
+             "latent_many_heads": O.latent_layer(40, 16, 16, 8, 48, scaling=YARN),        # more heads than one group of query rows
              "attention": O.attention_layer(4, 2, 32, 32, 16, window=20, keep_first=3, factor=3.0),
              "attention_wide": O.attention_layer(2, 1, 128, 128, 128, window=64, keep_first=0)}[kind]
     cfg = O.make_config([layer], vocab=8, width=W, eps=eps)
