@@ -234,9 +234,14 @@ __global__ __launch_bounds__(128) void sink_reduce_kernel(const float* __restric
   __syncthreads();
   const float gv = gate ? sigmoid_<FAST>(to_f32(gate[t * gate_row + head])) : 1.f;
   for (int d = threadIdx.x; d < dv; d += 128) {
-    float s = 0.f;
-    for (int z = 0; z < splits; ++z) s += wz[z] * p0[z * zs + d];
-    out[(t * H + head) * dv + d] = from_f32<T>(s / den * gv);
+    float s4[4] = {0.f, 0.f, 0.f, 0.f};               // four running sums: a row's loads do not wait for each other; the order is fixed
+    int z = 0;
+    for (; z + 4 <= splits; z += 4) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) s4[u] += wz[z + u] * p0[(z + u) * zs + d];
+    }
+    for (; z < splits; ++z) s4[z & 3] += wz[z] * p0[z * zs + d];
+    out[(t * H + head) * dv + d] = from_f32<T>(((s4[0] + s4[1]) + (s4[2] + s4[3])) / den * gv);
   }
 }
 
@@ -282,13 +287,21 @@ struct Segments {
 template <typename T>
 __global__ __launch_bounds__(NT) void rotate_norm_kernel(T* __restrict__ rows, int64_t stride, const int* __restrict__ positions, int64_t pos_stride,
                                                         Segments segs, float eps, int max_dim) {
-  extern __shared__ float head_lds[];               // [NW][2][max_dim]
+  extern __shared__ float head_lds[];               // [NW][2][max_dim], then cos [max_dim / 2], sin [max_dim / 2]
   const gbxm_head_segment sg = segs.s[blockIdx.y];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   float* in = head_lds + wave * 2 * max_dim;
   float* turned = in + max_dim;
+  float* cs_t = head_lds + NW * 2 * max_dim;
+  float* sn_t = cs_t + max_dim / 2 + 1;
   const float pos = static_cast<float>(positions[blockIdx.x * pos_stride]);
   const int half = sg.rot_dims / 2;
+  for (int i = threadIdx.x; i < half; i += NT) {    // the row's angles once, for all heads of the segment
+    float sn, cs;
+    sincosf(pos * sg.freq[i], &sn, &cs);
+    cs_t[i] = cs * sg.mult;
+    sn_t[i] = sn * sg.mult * sg.sign;
+  }
   for (int h0 = 0; h0 < sg.heads; h0 += NW) {
     const int head = h0 + wave;
     const bool live = head < sg.heads;
@@ -307,9 +320,7 @@ __global__ __launch_bounds__(NT) void rotate_norm_kernel(T* __restrict__ rows, i
         bool first;
         if (sg.interleaved) { i = idx >> 1; first = !(idx & 1); other = first ? c + 1 : c - 1; }
         else { first = idx < half; i = first ? idx : idx - half; other = first ? c + half : c - half; }
-        float sn, cs;
-        sincosf(pos * sg.freq[i], &sn, &cs);
-        sn *= sg.mult * sg.sign; cs *= sg.mult;
+        const float sn = sn_t[i], cs = cs_t[i];
         // (u, w) -> (u cos - w sin, w cos + u sin)
         v = first ? v * cs - in[other] * sn : v * cs + in[other] * sn;
       }
@@ -333,6 +344,26 @@ __global__ __launch_bounds__(NT) void stream_add_kernel(float* __restrict__ x, c
   float y = to_f32(a[i]);
   if (b) y += to_f32(b[i]);
   x[i] += y;
+}
+
+// x += a (+ b), then h = rms_norm(x) * w in the activation dtype: a parallel layer's stream update and the next layer's norm.
+template <typename T>
+__global__ __launch_bounds__(NT) void stream_add_norm_kernel(float* __restrict__ x, const T* __restrict__ a, const T* __restrict__ b,
+                                                            const float* __restrict__ w, T* __restrict__ h, int width, float eps) {
+  __shared__ float red[NW];
+  const int64_t t = blockIdx.x;
+  float* xr = x + t * width;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < width; c += NT) {
+    float y = to_f32(a[t * width + c]);
+    if (b) y += to_f32(b[t * width + c]);
+    const float v = xr[c] + y;
+    xr[c] = v;
+    ss += v * v;
+  }
+  ss = block_sum<NW>(ss, red);
+  const float r = 1.f / sqrtf(ss / width + eps);
+  for (int c = threadIdx.x; c < width; c += NT) h[t * width + c] = from_f32<T>(xr[c] * r * w[c]);      // (each thread re-reads what it wrote)
 }
 
 template <typename T>
@@ -393,6 +424,16 @@ int gbxm_stream_add(float* x, const void* a, const void* b, int64_t n, int32_t a
   return after_launch("stream_add");
 }
 
+int gbxm_stream_add_norm(float* x, const void* a, const void* b, const float* w, void* h, int64_t T_, int32_t width, float eps, int32_t act,
+                         void* stream) {
+  if (!act_ok(act) || !x || !a || !w || !h || T_ < 0 || width <= 0) return fail(GBXM_ERR_INVALID, "stream_add_norm: bad argument");
+  if (T_ == 0) return GBXM_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  GBXM_DISPATCH(act, (stream_add_norm_kernel<T><<<dim3(T_), NT, 0, s>>>(x, static_cast<const T*>(a), static_cast<const T*>(b), w, static_cast<T*>(h),
+                                                                          width, eps)));
+  return after_launch("stream_add_norm");
+}
+
 int gbxm_activate(void* z, int64_t n, int32_t kind, int32_t act, void* stream) {
   if (!act_ok(act) || !z || n < 0 || (kind != GBXM_ACT_RELU2 && kind != GBXM_ACT_GELU_TANH)) return fail(GBXM_ERR_INVALID, "activate: bad argument");
   if (n == 0) return GBXM_OK;
@@ -416,7 +457,7 @@ int gbxm_rotate_norm_heads(void* rows, int64_t T_, int64_t row_stride, const int
     sg.s[i] = g;
     max_dim = std::max(max_dim, g.head_dim);
   }
-  const size_t lds = static_cast<size_t>(NW) * 2 * max_dim * sizeof(float);
+  const size_t lds = (static_cast<size_t>(NW) * 2 * max_dim + 2 * (max_dim / 2 + 1)) * sizeof(float);
   if (lds > 60 * 1024) return fail(GBXM_ERR_UNSUPPORTED, "rotate_norm_heads: heads of %d channels", max_dim);
   if (T_ == 0) return GBXM_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);

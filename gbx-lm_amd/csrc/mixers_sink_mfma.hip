@@ -36,18 +36,16 @@ struct SinkTileArgs {
 };
 
 template <int DK, int DV>
-__global__ __launch_bounds__(256) void sink_tile_kernel(const SinkTileArgs a) {
+__device__ __forceinline__ void sink_tile(const SinkTileArgs& a, const int tile, unsigned char* lds) {
   constexpr int KT = 32;
   constexpr int KROW = DK * 2 + 16;          // +16 B: conflict-free 16-byte fragment reads
   constexpr int VROW = DV * 2 + 64;          // pitch = 16 dwords mod 64: the 4 rows of a transposed block land on disjoint banks
   constexpr int KS = DK / 16, DT = DV / 32;
-  __shared__ __attribute__((aligned(16))) unsigned char lds[KT * KROW + KT * VROW];
   unsigned char* kl = lds;
   unsigned char* vl = lds + KT * KROW;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 31, hb = lane >> 5;
-  const int tile = gridDim.x - 1 - blockIdx.x;               // a sequence's late tiles see the most keys: they are scheduled first
   const int b = a.tiles[2 * tile], tq = a.tiles[2 * tile + 1];
   const int head = blockIdx.y, kvh = head / (a.H / a.G);
   const int slot = a.seq[4 * b], pos0 = a.seq[4 * b + 1], n = a.seq[4 * b + 2], row0 = a.seq[4 * b + 3];
@@ -365,9 +363,19 @@ int launch_group(const SinkTileArgs& t, const gbxm_sink_attn_args& a, hipStream_
   return launch_sink_reduce(a, splits, s);
 }
 
+// A workgroup takes two query tiles, one from each end of the step's list: in a long causal prompt a late tile (many keys) and an
+// early one (few), so that workgroups carry about the same work however they are spread over the chip.
+template <int DK, int DV>
+__global__ __launch_bounds__(256, (DK + DV <= 320 ? 2 : 1)) void sink_tile_kernel(const SinkTileArgs a, const int n_tiles) {
+  __shared__ __attribute__((aligned(16))) unsigned char lds[32 * (DK * 2 + 16) + 32 * (DV * 2 + 64)];
+  const int first = n_tiles - 1 - blockIdx.x, second = blockIdx.x;
+  sink_tile<DK, DV>(a, first, lds);
+  if (second != first) sink_tile<DK, DV>(a, second, lds);
+}
+
 template <int DK, int DV>
 int launch(const SinkTileArgs& t, int n_tiles, hipStream_t s) {
-  sink_tile_kernel<DK, DV><<<dim3(n_tiles, t.H), 256, 0, s>>>(t);
+  sink_tile_kernel<DK, DV><<<dim3((n_tiles + 1) / 2, t.H), 256, 0, s>>>(t, n_tiles);
   return after_launch("sink_attention (tiles)");
 }
 
@@ -410,7 +418,7 @@ int launch_sink_tiles(const gbxm_sink_attn_args& a, hipStream_t s) {
 
 // values that are the leading channels of the key rows (same buffers, same strides): one staged tile serves both products
 static bool values_alias_keys(const gbxm_sink_attn_args& a) {
-  return a.G == 1 && a.dv <= a.dk && a.v_new == a.k_new && a.v_row == a.k_row &&
+  return a.G == 1 && a.dv <= a.dk && a.v_new == a.k_new && (a.T == 1 || a.v_row == a.k_row) &&     // (one row: its stride is never used)
          (!a.kcache || (a.vcache == a.kcache && a.vc_slot == a.kc_slot && a.vc_row == a.kc_row));
 }
 

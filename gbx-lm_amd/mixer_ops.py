@@ -162,6 +162,20 @@ def stream_add_(x: torch.Tensor, a: torch.Tensor, b: Optional[torch.Tensor] = No
     return x
 
 
+def stream_add_norm_(x: torch.Tensor, a: torch.Tensor, b: Optional[torch.Tensor], w: torch.Tensor, eps: float) -> torch.Tensor:
+    """x += a (+ b) in place, returns rms_norm(x) * w in the branches' dtype: one launch for a layer's update and the next layer's norm."""
+    act = _act(a, "a")
+    _f32(x, "x")
+    if x.dim() != 2 or a.shape != x.shape or not a.is_contiguous() or (b is not None and (b.shape != x.shape or b.dtype != a.dtype or not b.is_contiguous())):
+        raise ValueError("stream_add_norm_: contiguous branches of the stream's shape and one dtype")
+    if w.numel() != x.shape[1]:
+        raise ValueError("stream_add_norm_: one norm weight per channel")
+    h = torch.empty(x.shape, dtype=a.dtype, device=x.device)
+    _lib.check_mixers(_lib.mixers().gbxm_stream_add_norm(x.data_ptr(), a.data_ptr(), None if b is None else b.data_ptr(), _f32(w, "w").data_ptr(),
+                                                        h.data_ptr(), x.shape[0], x.shape[1], float(eps), act, _stream(x.device)))
+    return h
+
+
 _ACTIVATION = {"relu2": 1, "gelu_tanh": 2}
 
 

@@ -20,7 +20,7 @@ from torch import nn
 from ..batching import StepBatch
 from .base import BaseModelArgs
 from .feed_forward import DenseFeedForward
-from .residual import StreamRMSNorm, stream_add_
+from .residual import StreamRMSNorm, stream_add_, stream_add_norm_
 from .sink_attention import LatentAttention, RotatedValueWindowAttention
 from .step_model import RaggedStepModel
 
@@ -79,10 +79,14 @@ class Layer(nn.Module):
         self.mixer = _mixer(args, spec)
         self.mlp = _feed_forward(args, spec.get("mlp"))
 
-    def forward(self, x: torch.Tensor, act_dtype: torch.dtype, batch: StepBatch, cache) -> None:
-        """Updates the fp32 stream ``x`` in place."""
-        h = self.norm1(x, act_dtype)
-        stream_add_(x, self.mixer(h, batch, cache), None if self.mlp is None else self.mlp(h))
+    def forward(self, x: torch.Tensor, h: torch.Tensor, batch: StepBatch, cache, next_norm: Optional[StreamRMSNorm]) -> Optional[torch.Tensor]:
+        """``h`` = this layer's norm of the fp32 stream ``x``.  Updates ``x`` in place and returns the NEXT run's norm of it (the update
+        and that norm are one launch), or None after the last run."""
+        y, z = self.mixer(h, batch, cache), (None if self.mlp is None else self.mlp(h))
+        if next_norm is None:
+            stream_add_(x, y, z)
+            return None
+        return stream_add_norm_(x, y, z, next_norm)
 
 
 class RadenexModel(nn.Module):
@@ -114,9 +118,10 @@ class Model(RaggedStepModel):
     def forward_tokens(self, tokens: torch.Tensor, batch: StepBatch, caches) -> torch.Tensor:
         """One ragged step: tokens [T] -> fp32 stream [T, width] after the last layer run.  Positions are NOT advanced here."""
         x = self.model.embed(tokens)
-        act = self.lm_head.weight.dtype
-        for i, cache in zip(self._runs, caches):
-            self.model.layers[i](x, act, batch, cache)
+        layers, runs = self.model.layers, self._runs
+        h = layers[runs[0]].norm1(x, self.lm_head.weight.dtype) if runs else None
+        for n, (i, cache) in enumerate(zip(runs, caches)):
+            h = layers[i](x, h, batch, cache, layers[runs[n + 1]].norm1 if n + 1 < len(runs) else None)
             if self.trace_layers is not None:
                 self.trace_layers.append(x.clone())
         return x

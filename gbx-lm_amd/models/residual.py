@@ -53,3 +53,11 @@ def stream_add_(x: torch.Tensor, a: torch.Tensor, b: Optional[torch.Tensor] = No
         return M.stream_add_(x, a, b)
     y = a.float() if b is None else a.float() + b.float()
     return x.add_(y)
+
+
+def stream_add_norm_(x: torch.Tensor, a: torch.Tensor, b: Optional[torch.Tensor], norm: "StreamRMSNorm") -> torch.Tensor:
+    """``stream_add_`` followed by ``norm`` of the updated stream (the next layer's input), as one launch on the GPU."""
+    if x.is_cuda:
+        from .. import mixer_ops as M
+        return M.stream_add_norm_(x, a, b, norm.weight, norm.eps)
+    return norm(stream_add_(x, a, b), a.dtype)

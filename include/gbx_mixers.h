@@ -78,6 +78,9 @@ int gbxm_window_append(const void* qkv, int64_t row_stride, int32_t nq, int32_t 
 
 /* x[i] += a[i] (+ b[i]) in fp32 over n elements; a, b in the activation dtype (b may be null). */
 int gbxm_stream_add(float* x, const void* a, const void* b, int64_t n, int32_t act, void* stream);
+/* The same update of rows [T][width], then h[t] = rms_norm(x[t]) * w in the activation dtype (the next layer's input). */
+int gbxm_stream_add_norm(float* x, const void* a, const void* b, const float* w, void* h, int64_t T, int32_t width, float eps, int32_t act,
+                         void* stream);
 /* In place on n elements, fp32 arithmetic: kind 1 = relu(z)^2, 2 = gelu in its tanh form. */
 #define GBXM_ACT_RELU2 1
 #define GBXM_ACT_GELU_TANH 2

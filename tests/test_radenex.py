@@ -283,6 +283,15 @@ def test_feed_forward_and_stream_update(device, dtype):
     assert torch.allclose(got, x + (a.float() + b.float()), atol=1e-6)
     got = stream_add_(x.clone().to(device), a.to(device), None).cpu()
     assert torch.allclose(got, x + a.float(), atol=1e-6)
+    from gbx_lm_amd.models.residual import StreamRMSNorm, stream_add_norm_
+    norm = StreamRMSNorm(300, 1e-5)
+    norm.weight.copy_(torch.rand(300, generator=g) + 0.5)
+    norm = norm.to(device)
+    xs = x.clone().to(device)
+    h = stream_add_norm_(xs, a.to(device), b.to(device), norm)
+    want_x = x.double() + (a.double() + b.double())
+    assert torch.allclose(xs.cpu().double(), want_x, atol=1e-6) and h.dtype == dtype
+    assert O.rel_err(h.float(), O.rms(want_x, 1e-5, norm.weight.cpu().double())) < (1e-6 if dtype == torch.float32 else 1e-2)
 
 
 @pytest.mark.parametrize("device", DEVICES)
