@@ -370,6 +370,7 @@ def mixers() -> ctypes.CDLL:
         L.gbxm_window_append.argtypes = [p, i64, i32, i32, i32, p, p, p, p, i64, i32, i32, p]
         L.gbxm_stream_add.argtypes = [p, p, p, i64, i32, p]
         L.gbxm_activate.argtypes = [p, i64, i32, i32, p]
+        L.gbxm_head_project.argtypes = [p, i64, i64, p, p, i64, i64, i64, i32, i32, i32, i32, i32, p]
         L.gbxm_stream_add_norm.argtypes = [p, p, p, p, p, i64, i32, f32, i32, p]
         L.gbxm_rotate_norm_heads.argtypes = [p, i64, i64, p, i64, ctypes.POINTER(HeadSegment), i32, f32, i32, p]
         L.gbxm_slot_append.argtypes = [p, i64, i32, p, i64, i32, p, p, p, p, i64, i32, i32, i32, p]

@@ -366,6 +366,31 @@ __global__ __launch_bounds__(NT) void stream_add_norm_kernel(float* __restrict__
   for (int c = threadIdx.x; c < width; c += NT) h[t * width + c] = from_f32<T>(xr[c] * r * w[c]);      // (each thread re-reads what it wrote)
 }
 
+// out[t][h][j] = sum_i in[t][h][i] w[h][i][j] for j < n_out, then out[t][h][n_out + c] = in[t][h][n_in + c] for c < n_tail: a small
+// matrix of its own per head, applied to few rows (single-row steps): one workgroup per (row, head), the head's input in LDS,
+// threads across the outputs (coalesced reads of w), fp32 sums.
+template <typename T>
+__global__ __launch_bounds__(NT) void head_project_kernel(const T* __restrict__ in, int64_t in_row, int64_t in_head, const T* __restrict__ w,
+                                                         T* __restrict__ out, int64_t out_row, int64_t out_head, int n_in, int n_out, int n_tail) {
+  extern __shared__ float xin[];                   // [n_in]
+  const T* ip = in + blockIdx.x * in_row + blockIdx.y * in_head;
+  T* op = out + blockIdx.x * out_row + blockIdx.y * out_head;
+  const T* wp = w + static_cast<int64_t>(blockIdx.y) * n_in * n_out;
+  for (int i = threadIdx.x; i < n_in; i += NT) xin[i] = to_f32(ip[i]);
+  __syncthreads();
+  for (int j = threadIdx.x; j < n_out; j += NT) {
+    float s4[4] = {0.f, 0.f, 0.f, 0.f};
+    int i = 0;
+    for (; i + 4 <= n_in; i += 4) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) s4[u] += xin[i + u] * to_f32(wp[static_cast<int64_t>(i + u) * n_out + j]);
+    }
+    for (; i < n_in; ++i) s4[i & 3] += xin[i] * to_f32(wp[static_cast<int64_t>(i) * n_out + j]);
+    op[j] = from_f32<T>((s4[0] + s4[1]) + (s4[2] + s4[3]));
+  }
+  for (int c = threadIdx.x; c < n_tail; c += NT) op[n_out + c] = ip[n_in + c];
+}
+
 template <typename T>
 __global__ __launch_bounds__(NT) void activate_kernel(T* __restrict__ z, int64_t n, int kind) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * NT + threadIdx.x;
@@ -432,6 +457,19 @@ int gbxm_stream_add_norm(float* x, const void* a, const void* b, const float* w,
   GBXM_DISPATCH(act, (stream_add_norm_kernel<T><<<dim3(T_), NT, 0, s>>>(x, static_cast<const T*>(a), static_cast<const T*>(b), w, static_cast<T*>(h),
                                                                           width, eps)));
   return after_launch("stream_add_norm");
+}
+
+int gbxm_head_project(const void* in, int64_t in_row, int64_t in_head, const void* w, void* out, int64_t out_row, int64_t out_head, int64_t T_,
+                      int32_t H, int32_t n_in, int32_t n_out, int32_t n_tail, int32_t act, void* stream) {
+  if (!act_ok(act) || !in || !w || !out || T_ < 0 || H < 1 || H > 65535 || n_in < 1 || n_out < 1 || n_tail < 0)
+    return fail(GBXM_ERR_INVALID, "head_project: bad argument");
+  if (n_in > 12 * 1024) return fail(GBXM_ERR_UNSUPPORTED, "head_project: %d input channels per head", n_in);
+  if (T_ == 0) return GBXM_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  GBXM_DISPATCH(act, (head_project_kernel<T><<<dim3(T_, H), NT, n_in * sizeof(float), s>>>(static_cast<const T*>(in), in_row, in_head,
+                                                                                           static_cast<const T*>(w), static_cast<T*>(out), out_row,
+                                                                                           out_head, n_in, n_out, n_tail)));
+  return after_launch("head_project");
 }
 
 int gbxm_activate(void* z, int64_t n, int32_t kind, int32_t act, void* stream) {

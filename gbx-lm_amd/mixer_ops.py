@@ -176,6 +176,20 @@ def stream_add_norm_(x: torch.Tensor, a: torch.Tensor, b: Optional[torch.Tensor]
     return h
 
 
+def head_project(x: torch.Tensor, w: torch.Tensor, n_tail: int = 0) -> torch.Tensor:
+    """x [T, H, n_in + n_tail] (unit channel stride), w [H, n_in, n_out] -> [T, H, n_out + n_tail]: every head's own matrix on its
+    first n_in channels, the tail copied through.  For the few rows of decode steps (one workgroup per row and head)."""
+    act = _act(x, "x")
+    t, heads, width = x.shape
+    n_in, n_out = w.shape[1], w.shape[2]
+    if w.shape[0] != heads or width != n_in + n_tail or x.stride(2) != 1 or w.dtype != x.dtype or not w.is_contiguous():
+        raise ValueError("head_project: operands do not fit")
+    out = torch.empty((t, heads, n_out + n_tail), dtype=x.dtype, device=x.device)
+    _lib.check_mixers(_lib.mixers().gbxm_head_project(x.data_ptr(), x.stride(0), x.stride(1), w.data_ptr(), out.data_ptr(), out.stride(0), out.stride(1),
+                                                     t, heads, n_in, n_out, n_tail, act, _stream(x.device)))
+    return out
+
+
 _ACTIVATION = {"relu2": 1, "gelu_tanh": 2}
 
 

@@ -136,6 +136,17 @@ def sink_attend(q: torch.Tensor, k_new: torch.Tensor, v_new: torch.Tensor, cache
     return out
 
 
+def head_project(x: torch.Tensor, w: torch.Tensor, n_tail: int = 0) -> torch.Tensor:
+    """x [T, H, n_in + n_tail], w [H, n_in, n_out] -> [T, H, n_out + n_tail]: each head's own matrix on its first n_in channels, the
+    remaining channels copied through.  Few GPU rows: one HIP launch; else a batched matrix product."""
+    if x.is_cuda and x.shape[0] <= 32:
+        from .. import mixer_ops as M
+        return M.head_project(x, w, n_tail)
+    n_in = w.shape[1]
+    y = torch.bmm(x[:, :, :n_in].transpose(0, 1), w).transpose(0, 1)
+    return torch.cat([y, x[:, :, n_in:]], dim=-1) if n_tail else y.contiguous()
+
+
 def cache_append(cache: SlotKVCache, k_rows: torch.Tensor, v_rows: Optional[torch.Tensor], batch) -> None:
     """The step's key rows [T, k_width] (and value rows) into the table, after every query of the step has attended."""
     if k_rows.is_cuda:
@@ -243,11 +254,9 @@ class LatentAttention(nn.Module):
             keys[:, :, d:] = latent[:, None, rank:]
             ctx = sink_attend(q, keys, kv[:, self.nq:].view(t, hd, dv), None, batch, self.scale, None, 0, self.sink, gate)
         else:
-            qa = torch.empty((t, hd, self.nl), dtype=y.dtype, device=y.device)
-            qa[:, :, :rank] = torch.bmm(q[:, :, :d].transpose(0, 1), self.uk_heads).transpose(0, 1)
-            qa[:, :, rank:] = q[:, :, d:]
+            qa = head_project(q, self.uk_heads, r)                                 # W_uk^T q | rotated part, per head
             mixed = sink_attend(qa, latent.view(t, 1, self.nl), latent[:, :rank].view(t, 1, rank), cache, batch, self.scale, None, 0,
                                 self.sink, gate)
-            ctx = torch.bmm(mixed.view(t, hd, rank).transpose(0, 1), self.uv_heads_t).transpose(0, 1).reshape(t, hd * dv)
+            ctx = head_project(mixed.view(t, hd, rank), self.uv_heads_t).view(t, hd * dv)
         cache_append(cache, latent, None, batch)
         return F.linear(ctx, self.o.weight)

@@ -81,6 +81,10 @@ int gbxm_stream_add(float* x, const void* a, const void* b, int64_t n, int32_t a
 /* The same update of rows [T][width], then h[t] = rms_norm(x[t]) * w in the activation dtype (the next layer's input). */
 int gbxm_stream_add_norm(float* x, const void* a, const void* b, const float* w, void* h, int64_t T, int32_t width, float eps, int32_t act,
                          void* stream);
+/* A matrix per head on few rows: out[t][h][j] = sum_i in[t][h][i] w[h][i][j] (j < n_out), then n_tail channels copied from
+ * in[t][h][n_in ..] to out[t][h][n_out ..].  Strides in elements; w is [H][n_in][n_out]. */
+int gbxm_head_project(const void* in, int64_t in_row, int64_t in_head, const void* w, void* out, int64_t out_row, int64_t out_head, int64_t T,
+                      int32_t H, int32_t n_in, int32_t n_out, int32_t n_tail, int32_t act, void* stream);
 /* In place on n elements, fp32 arithmetic: kind 1 = relu(z)^2, 2 = gelu in its tanh form. */
 #define GBXM_ACT_RELU2 1
 #define GBXM_ACT_GELU_TANH 2

@@ -296,6 +296,22 @@ def test_feed_forward_and_stream_update(device, dtype):
 
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows", [1, 7, 40])
+def test_head_project(device, dtype, rows):
+    """Every head's own matrix on the head's leading channels, the rest copied through (few rows: one launch; more: batched product)."""
+    g = torch.Generator().manual_seed(rows)
+    heads, n_in, n_out, tail = 5, 37, 300, 6
+    x = torch.randn((rows, heads * (n_in + tail) + 3), generator=g).to(dtype)[:, :heads * (n_in + tail)].view(rows, heads, n_in + tail)   # strided rows
+    w = (torch.randn((heads, n_in, n_out), generator=g) / 6).to(dtype)
+    want = torch.cat([torch.einsum("thi,hio->tho", x[..., :n_in].double(), w.double()), x[..., n_in:].double()], dim=-1)
+    got = SA.head_project(x.to(device), w.to(device), tail)
+    assert got.shape == want.shape and O.rel_err(got.float().reshape(rows, -1), want.reshape(rows, -1)) < (1e-6 if dtype == torch.float32 else 1e-2)
+    got = SA.head_project(x[..., :n_in].to(device), w.to(device))
+    assert O.rel_err(got.float().reshape(rows, -1), want[..., :n_out].reshape(rows, -1)) < (1e-6 if dtype == torch.float32 else 1e-2)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("kind", ["latent", "attention", "latent_odd", "attention_wide", "latent_wide", "latent_many_heads"])
 def test_mixers_alone(device, dtype, kind):
     """One mixer module with random weights: a whole prompt (keys and values formed per head), then token by token and in portions
