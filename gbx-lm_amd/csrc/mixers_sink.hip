@@ -391,6 +391,58 @@ __global__ __launch_bounds__(NT) void head_project_kernel(const T* __restrict__ 
   for (int c = threadIdx.x; c < n_tail; c += NT) op[n_out + c] = ip[n_in + c];
 }
 
+// The same with 16-byte loads of w: a thread owns a run of PER outputs and every IS-th input channel (IS = 256 / (outputs / PER):
+// all threads stream w, many loads in flight each); the IS partial sums of an output meet in LDS in a fixed order.
+template <typename T>
+__global__ __launch_bounds__(NT) void head_project_vec_kernel(const T* __restrict__ in, int64_t in_row, int64_t in_head, const T* __restrict__ w,
+                                                             T* __restrict__ out, int64_t out_row, int64_t out_head, int n_in, int n_out, int n_tail) {
+  constexpr int PER = 16 / sizeof(T);
+  extern __shared__ float xin[];                   // [n_in], then the partial sums [NT * PER]
+  float* red = xin + n_in;
+  const T* ip = in + blockIdx.x * in_row + blockIdx.y * in_head;
+  T* op = out + blockIdx.x * out_row + blockIdx.y * out_head;
+  const T* wp = w + static_cast<int64_t>(blockIdx.y) * n_in * n_out;
+  const int tid = threadIdx.x;
+  for (int i = tid; i < n_in; i += NT) xin[i] = to_f32(ip[i]);
+  for (int jb = 0; jb < n_out; jb += NT * PER) {
+    const int jn = min(n_out - jb, NT * PER);
+    const int JC = jn / PER, IS = NT / JC;
+    const int jc = tid % JC, is = tid / JC;
+    float acc[PER];
+#pragma unroll
+    for (int u = 0; u < PER; ++u) acc[u] = 0.f;
+    __syncthreads();                               // xin is there; red is free
+    if (is < IS) {
+      const T* col = wp + jb + jc * PER;
+#pragma unroll 8
+      for (int i = is; i < n_in; i += IS) {
+        const uint4 raw = *reinterpret_cast<const uint4*>(col + static_cast<int64_t>(i) * n_out);
+        const float x = xin[i];
+        if constexpr (sizeof(T) == 2) {
+          const unsigned u4[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            acc[2 * u] += x * __uint_as_float(u4[u] << 16);
+            acc[2 * u + 1] += x * __uint_as_float(u4[u] & 0xFFFF0000u);
+          }
+        } else {
+          acc[0] += x * __uint_as_float(raw.x); acc[1] += x * __uint_as_float(raw.y);
+          acc[2] += x * __uint_as_float(raw.z); acc[3] += x * __uint_as_float(raw.w);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < PER; ++u) red[is * jn + jc * PER + u] = acc[u];
+    }
+    __syncthreads();
+    for (int j = tid; j < jn; j += NT) {
+      float s = 0.f;
+      for (int k = 0; k < IS; ++k) s += red[k * jn + j];
+      op[jb + j] = from_f32<T>(s);
+    }
+  }
+  for (int c = tid; c < n_tail; c += NT) op[n_out + c] = ip[n_in + c];
+}
+
 template <typename T>
 __global__ __launch_bounds__(NT) void activate_kernel(T* __restrict__ z, int64_t n, int kind) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * NT + threadIdx.x;
@@ -466,6 +518,13 @@ int gbxm_head_project(const void* in, int64_t in_row, int64_t in_head, const voi
   if (n_in > 12 * 1024) return fail(GBXM_ERR_UNSUPPORTED, "head_project: %d input channels per head", n_in);
   if (T_ == 0) return GBXM_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  const int per = act == GBXM_BF16 ? 8 : 4;
+  if (n_out % per == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0) {
+    GBXM_DISPATCH(act, (head_project_vec_kernel<T><<<dim3(T_, H), NT, (n_in + NT * per) * sizeof(float), s>>>(
+                           static_cast<const T*>(in), in_row, in_head, static_cast<const T*>(w), static_cast<T*>(out), out_row, out_head, n_in, n_out,
+                           n_tail)));
+    return after_launch("head_project");
+  }
   GBXM_DISPATCH(act, (head_project_kernel<T><<<dim3(T_, H), NT, n_in * sizeof(float), s>>>(static_cast<const T*>(in), in_row, in_head,
                                                                                            static_cast<const T*>(w), static_cast<T*>(out), out_row,
                                                                                            out_head, n_in, n_out, n_tail)));

@@ -308,6 +308,11 @@ def test_head_project(device, dtype, rows):
     assert got.shape == want.shape and O.rel_err(got.float().reshape(rows, -1), want.reshape(rows, -1)) < (1e-6 if dtype == torch.float32 else 1e-2)
     got = SA.head_project(x[..., :n_in].to(device), w.to(device))
     assert O.rel_err(got.float().reshape(rows, -1), want[..., :n_out].reshape(rows, -1)) < (1e-6 if dtype == torch.float32 else 1e-2)
+    w2 = (torch.randn((heads, n_in, 2600), generator=g) / 6).to(dtype)                    # 16-byte rows of w, more outputs than one pass
+    got = SA.head_project(x.to(device), w2.to(device), tail)
+    want2 = torch.einsum("thi,hio->tho", x[..., :n_in].double(), w2.double())
+    assert O.rel_err(got[..., :2600].float().reshape(rows, -1), want2.reshape(rows, -1)) < (1e-6 if dtype == torch.float32 else 1e-2)
+    assert torch.equal(got[..., 2600:].cpu(), x[..., n_in:])
 
 
 @pytest.mark.parametrize("device", DEVICES)
