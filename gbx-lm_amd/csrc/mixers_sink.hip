@@ -443,15 +443,36 @@ __global__ __launch_bounds__(NT) void head_project_vec_kernel(const T* __restric
   for (int c = tid; c < n_tail; c += NT) op[n_out + c] = ip[n_in + c];
 }
 
+__device__ __forceinline__ float activation(float v, int kind) {
+  if (kind == GBXM_ACT_RELU2) { const float r = fmaxf(v, 0.f); return r * r; }
+  return 0.5f * v * (1.f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
+}
+
 template <typename T>
 __global__ __launch_bounds__(NT) void activate_kernel(T* __restrict__ z, int64_t n, int kind) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * NT + threadIdx.x;
   if (i >= n) return;
-  const float v = to_f32(z[i]);
-  float y;
-  if (kind == GBXM_ACT_RELU2) { const float r = fmaxf(v, 0.f); y = r * r; }
-  else y = 0.5f * v * (1.f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
-  z[i] = from_f32<T>(y);
+  z[i] = from_f32<T>(activation(to_f32(z[i]), kind));
+}
+
+// 16 bytes per thread (n a multiple of the vector, base 16-byte aligned)
+template <typename T>
+__global__ __launch_bounds__(NT) void activate_vec_kernel(T* __restrict__ z, int64_t n_vec, int kind) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * NT + threadIdx.x;
+  if (i >= n_vec) return;
+  uint4* p = reinterpret_cast<uint4*>(z) + i;
+  uint4 raw = *p;
+  unsigned u[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    if constexpr (sizeof(T) == 2) {
+      const float lo = activation(__uint_as_float(u[k] << 16), kind), hi = activation(__uint_as_float(u[k] & 0xFFFF0000u), kind);
+      u[k] = static_cast<unsigned>(f32_to_bf16(lo)) | (static_cast<unsigned>(f32_to_bf16(hi)) << 16);
+    } else {
+      u[k] = __float_as_uint(activation(__uint_as_float(u[k]), kind));
+    }
+  }
+  *p = uint4{u[0], u[1], u[2], u[3]};
 }
 
 template <typename T>
@@ -535,6 +556,12 @@ int gbxm_activate(void* z, int64_t n, int32_t kind, int32_t act, void* stream) {
   if (!act_ok(act) || !z || n < 0 || (kind != GBXM_ACT_RELU2 && kind != GBXM_ACT_GELU_TANH)) return fail(GBXM_ERR_INVALID, "activate: bad argument");
   if (n == 0) return GBXM_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  const int per = act == GBXM_BF16 ? 8 : 4;
+  if (n % per == 0 && reinterpret_cast<uintptr_t>(z) % 16 == 0) {
+    const int64_t nv = n / per;
+    GBXM_DISPATCH(act, (activate_vec_kernel<T><<<dim3((nv + NT - 1) / NT), NT, 0, s>>>(static_cast<T*>(z), nv, kind)));
+    return after_launch("activate");
+  }
   GBXM_DISPATCH(act, (activate_kernel<T><<<dim3((n + NT - 1) / NT), NT, 0, s>>>(static_cast<T*>(z), n, kind)));
   return after_launch("activate");
 }
