@@ -49,6 +49,10 @@ template <bool FAST> __device__ __forceinline__ float tanh_(float x) {
 }
 template <bool FAST> __device__ __forceinline__ float log1p_(float x) { if constexpr (FAST) return __logf(1.f + x); else return log1pf(x); }
 
+// floats per (split, row, head) of the key-split partial sums of softmax attention: dv sums padded to a multiple of four (rows stay
+// 16-byte aligned), then two more pairs of which the last holds (running maximum, denominator)
+__host__ __device__ __forceinline__ int partial_width(int dv) { return (dv + 3) / 4 * 4 + 4; }
+
 extern thread_local char g_err[512];
 int fail(int code, const char* fmt, ...);
 int hip_fail(hipError_t e, const char* what);

@@ -183,16 +183,17 @@ __global__ __launch_bounds__(NT) void sink_rows_kernel(const T* __restrict__ q, 
   }
   __syncthreads();
   if (splits > 1) {
-    float* prow = partial + ((static_cast<int64_t>(blockIdx.z) * gridDim.x + t) * g.H + head0) * (g.dv + 2);
+    const int pw = partial_width(g.dv);
+    float* prow = partial + ((static_cast<int64_t>(blockIdx.z) * gridDim.x + t) * g.H + head0) * pw;
     for (int i = threadIdx.x; i < nr * g.dv; i += NT) {
       float s = 0.f;
 #pragma unroll
       for (int w = 0; w < NW; ++w) s += sums[w * rc * g.dv + i];
-      prow[(i / g.dv) * (g.dv + 2) + i % g.dv] = s;
+      prow[(i / g.dv) * pw + i % g.dv] = s;
     }
     if (threadIdx.x < nr) {
-      prow[threadIdx.x * (g.dv + 2) + g.dv] = ml[threadIdx.x];
-      prow[threadIdx.x * (g.dv + 2) + g.dv + 1] = ll[threadIdx.x];
+      prow[threadIdx.x * pw + pw - 2] = ml[threadIdx.x];
+      prow[threadIdx.x * pw + pw - 1] = ll[threadIdx.x];
     }
     return;
   }
@@ -209,39 +210,52 @@ __global__ __launch_bounds__(NT) void sink_rows_kernel(const T* __restrict__ q, 
 }
 
 // One workgroup per (row, head): joins the key splits' (sum, maximum, denominator) in split order, adds the sink, applies the gate.
+// Rows of `partial` are partial_width(dv) floats (the sums, padding to a multiple of four, maximum, denominator), so a thread
+// reads four channels at once; the two halves of the workgroup take the even and the odd splits and meet in LDS.
 template <typename T, bool FAST>
-__global__ __launch_bounds__(128) void sink_reduce_kernel(const float* __restrict__ partial, T* __restrict__ out, const float* __restrict__ sink,
+__global__ __launch_bounds__(256) void sink_reduce_kernel(const float* __restrict__ partial, T* __restrict__ out, const float* __restrict__ sink,
                                                          const T* __restrict__ gate, int64_t gate_row, int64_t T_, int H, int dv, int splits) {
   __shared__ float wz[64];
   __shared__ float den;
+  __shared__ float4 other[128];
   const int64_t t = blockIdx.x;
-  const int head = blockIdx.y;
-  const int64_t zs = T_ * H * (dv + 2);
-  const float* p0 = partial + (t * H + head) * (dv + 2);
+  const int head = blockIdx.y, pw = partial_width(dv);
+  const int64_t zs = T_ * H * pw;
+  const float* p0 = partial + (t * H + head) * pw;
   if (threadIdx.x < 64) {
     const int z = threadIdx.x;
-    const float m = z < splits ? p0[z * zs + dv] : -INFINITY;
+    const float m = z < splits ? p0[z * zs + pw - 2] : -INFINITY;
     float top = m;
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) top = fmaxf(top, __shfl_xor(top, o, 64));
     if (sink) top = fmaxf(top, sink[head]);
     const float w = z < splits ? exp_<FAST>(m - top) : 0.f;
     wz[z] = w;
-    float l = z < splits ? w * p0[z * zs + dv + 1] : 0.f;
+    float l = z < splits ? w * p0[z * zs + pw - 1] : 0.f;
     l = wave_sum(l);
     if (z == 0) den = l + (sink ? exp_<FAST>(sink[head] - top) : 0.f);
   }
   __syncthreads();
-  const float gv = gate ? sigmoid_<FAST>(to_f32(gate[t * gate_row + head])) : 1.f;
-  for (int d = threadIdx.x; d < dv; d += 128) {
-    float s4[4] = {0.f, 0.f, 0.f, 0.f};               // four running sums: a row's loads do not wait for each other; the order is fixed
-    int z = 0;
-    for (; z + 4 <= splits; z += 4) {
-#pragma unroll
-      for (int u = 0; u < 4; ++u) s4[u] += wz[z + u] * p0[(z + u) * zs + d];
+  const float f = (gate ? sigmoid_<FAST>(to_f32(gate[t * gate_row + head])) : 1.f) / den;
+  const int half = threadIdx.x >> 7, q = threadIdx.x & 127;
+  for (int d0 = 0; d0 < dv; d0 += 512) {
+    const int d = d0 + 4 * q;
+    float4 s = float4{0.f, 0.f, 0.f, 0.f};
+    if (d < dv)
+#pragma unroll 4
+      for (int z = half; z < splits; z += 2) {
+        const float4 v = *reinterpret_cast<const float4*>(p0 + z * zs + d);      // (channels past dv inside the last four are padding)
+        const float w = wz[z];
+        s.x += w * v.x; s.y += w * v.y; s.z += w * v.z; s.w += w * v.w;
+      }
+    __syncthreads();
+    if (half) other[q] = s;
+    __syncthreads();
+    if (!half && d < dv) {
+      const float4 u = other[q];
+      const float r[4] = {(s.x + u.x) * f, (s.y + u.y) * f, (s.z + u.z) * f, (s.w + u.w) * f};
+      for (int c = 0; c < 4 && d + c < dv; ++c) out[(t * H + head) * dv + d + c] = from_f32<T>(r[c]);
     }
-    for (; z < splits; ++z) s4[z & 3] += wz[z] * p0[z * zs + d];
-    out[(t * H + head) * dv + d] = from_f32<T>(((s4[0] + s4[1]) + (s4[2] + s4[3])) / den * gv);
   }
 }
 
@@ -273,7 +287,7 @@ int launch_rows(const gbxm_sink_attn_args& a, const SinkGeo& g, int rc, int chun
     sink_rows_kernel<T, FAST, true><<<grid, NT, lds, s>>>(q, kn, vn, kc, vc, a.seq, a.tok, out, a.sink, gate, g, rc, splits, part);
   else
     sink_rows_kernel<T, FAST, false><<<grid, NT, lds, s>>>(q, kn, vn, kc, vc, a.seq, a.tok, out, a.sink, gate, g, rc, splits, part);
-  if (splits > 1) sink_reduce_kernel<T, FAST><<<dim3(a.T, a.H), 128, 0, s>>>(part, out, a.sink, gate, a.gate_row, a.T, a.H, a.dv, splits);
+  if (splits > 1) sink_reduce_kernel<T, FAST><<<dim3(a.T, a.H), 256, 0, s>>>(part, out, a.sink, gate, a.gate_row, a.T, a.H, a.dv, splits);
   return after_launch("sink_attention (rows)");
 }
 
@@ -498,7 +512,7 @@ int launch_sink_group(const gbxm_sink_attn_args& a, hipStream_t s);     // the s
 bool sink_tiles_shape(int dk, int dv);
 
 int launch_sink_reduce(const gbxm_sink_attn_args& a, int splits, hipStream_t s) {
-  sink_reduce_kernel<bf16_t, true><<<dim3(a.T, a.H), 128, 0, s>>>(static_cast<const float*>(a.partial), static_cast<bf16_t*>(a.out), a.sink,
+  sink_reduce_kernel<bf16_t, true><<<dim3(a.T, a.H), 256, 0, s>>>(static_cast<const float*>(a.partial), static_cast<bf16_t*>(a.out), a.sink,
                                                                   static_cast<const bf16_t*>(a.gate), a.gate_row, a.T, a.H, a.dv, splits);
   return after_launch("sink_attention (join of key splits)");
 }

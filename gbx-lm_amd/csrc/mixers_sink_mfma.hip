@@ -209,9 +209,16 @@ __global__ __launch_bounds__(256) void sink_group_kernel(const SinkTileArgs a, c
   constexpr int KROW = DK * 2 + 16;
   constexpr int VROW = ALIAS ? KROW : DV * 2 + 64;
   constexpr int KS = DK / 16, DT = DV / 32, DTW = (DT + 3) / 4;
-  __shared__ __attribute__((aligned(16))) unsigned char lds[KT * KROW + (ALIAS ? 0 : KT * VROW)];
+  // long rows: the channels of the score product are shared out over the four waves (a quarter of the dependent matrix-core steps
+  // and of the query fragments each); the four partial score tiles meet in LDS and every wave adds them in the same order, so all
+  // waves hold identical scores.  The registers this frees hold the next key tile while the current one is computed.
+  constexpr bool SPLITK = KS >= 16;
+  constexpr int KSW = SPLITK ? (KS + 3) / 4 : KS;
+  constexpr int TILE_BYTES = KT * KROW + (ALIAS ? 0 : KT * VROW);
+  __shared__ __attribute__((aligned(16))) unsigned char lds[TILE_BYTES + (SPLITK ? 4 * 16 * 64 * 4 : 0)];
   unsigned char* kl = lds;
   unsigned char* vl = ALIAS ? lds : lds + KT * KROW;
+  float* sred = reinterpret_cast<float*>(lds + TILE_BYTES);            // [4 waves][16][64 lanes]
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 31, hb = lane >> 5;
@@ -224,13 +231,14 @@ __global__ __launch_bounds__(256) void sink_group_kernel(const SinkTileArgs a, c
   const int slot = a.seq[4 * b], pos0 = a.seq[4 * b + 1], row0 = a.seq[4 * b + 3];
   const int W = a.window;
 
-  u32x4 qf[KS];
+  const int ks0 = SPLITK ? wave * KSW : 0;                              // this wave's steps of the score product: ks0 .. ks0 + KSW - 1
+  u32x4 qf[KSW];
   {
     const bf16_t* qp = a.q + t * a.q_row + head * a.q_head;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      const int c = ks * 16 + hb * 8;
-      qf[ks] = c < a.dk ? *reinterpret_cast<const u32x4*>(qp + c) : u32x4{0, 0, 0, 0};
+    for (int i = 0; i < KSW; ++i) {
+      const int c = (ks0 + i) * 16 + hb * 8;
+      qf[i] = (ks0 + i < KS && c < a.dk) ? *reinterpret_cast<const u32x4*>(qp + c) : u32x4{0, 0, 0, 0};
     }
   }
   f32x16 o[DTW];
@@ -258,26 +266,60 @@ __global__ __launch_bounds__(256) void sink_group_kernel(const SinkTileArgs a, c
   const unsigned char* vbase = vl + (4 * hb + ((lane >> 2) & 3)) * VROW + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
   const unsigned char* kbase = kl + r * KROW + hb * 16;
 
-  for (int it = static_cast<int>(blockIdx.z) * KT; it < total; it += KT * splits) {
-    __syncthreads();                                          // the previous tile has been consumed
-    for (int p = tid; p < KT * (DK / 8); p += 256) {
-      const int row = p / (DK / 8), c = p % (DK / 8), iv = it + row;
-      u32x4 v = u32x4{0, 0, 0, 0};
-      if (iv < total && c * 8 < a.dk) v = *reinterpret_cast<const u32x4*>(krow(pos_of(iv)) + c * 8);
-      *reinterpret_cast<u32x4*>(kl + row * KROW + c * 16) = v;
+  // a key (and value) tile: global -> registers -> LDS; with SPLITK the registers are filled one tile ahead
+  constexpr int KP = (KT * (DK / 8) + 255) / 256, VP = ALIAS ? 1 : (KT * (DV / 8) + 255) / 256;
+  u32x4 kr[KP], vr[VP];
+  auto fetch = [&](int it) {
+#pragma unroll
+    for (int i = 0; i < KP; ++i) {
+      const int p = tid + 256 * i, row = p / (DK / 8), c = p % (DK / 8), iv = it + row;
+      kr[i] = u32x4{0, 0, 0, 0};
+      if (p < KT * (DK / 8) && iv < total && c * 8 < a.dk) kr[i] = *reinterpret_cast<const u32x4*>(krow(pos_of(iv)) + c * 8);
     }
     if constexpr (!ALIAS) {
-      for (int p = tid; p < KT * (DV / 8); p += 256) {
-        const int row = p / (DV / 8), c = p % (DV / 8), iv = it + row;
-        u32x4 v = u32x4{0, 0, 0, 0};
-        if (iv < total && c * 8 < a.dv) v = *reinterpret_cast<const u32x4*>(vrow(pos_of(iv)) + c * 8);
-        *reinterpret_cast<u32x4*>(vl + row * VROW + c * 16) = v;
+#pragma unroll
+      for (int i = 0; i < VP; ++i) {
+        const int p = tid + 256 * i, row = p / (DV / 8), c = p % (DV / 8), iv = it + row;
+        vr[i] = u32x4{0, 0, 0, 0};
+        if (p < KT * (DV / 8) && iv < total && c * 8 < a.dv) vr[i] = *reinterpret_cast<const u32x4*>(vrow(pos_of(iv)) + c * 8);
       }
     }
+  };
+  auto stage = [&]() {
+#pragma unroll
+    for (int i = 0; i < KP; ++i) {
+      const int p = tid + 256 * i;
+      if (p < KT * (DK / 8)) *reinterpret_cast<u32x4*>(kl + (p / (DK / 8)) * KROW + (p % (DK / 8)) * 16) = kr[i];
+    }
+    if constexpr (!ALIAS) {
+#pragma unroll
+      for (int i = 0; i < VP; ++i) {
+        const int p = tid + 256 * i;
+        if (p < KT * (DV / 8)) *reinterpret_cast<u32x4*>(vl + (p / (DV / 8)) * VROW + (p % (DV / 8)) * 16) = vr[i];
+      }
+    }
+  };
+
+  const int it0 = static_cast<int>(blockIdx.z) * KT, step = KT * splits;
+  if (SPLITK && it0 < total) fetch(it0);
+  for (int it = it0; it < total; it += step) {
+    if constexpr (!SPLITK) fetch(it);
+    __syncthreads();                                          // the previous tile (and its partial scores) have been consumed
+    stage();
     __syncthreads();
+    if (SPLITK && it + step < total) fetch(it + step);        // the next tile travels while this one is computed
     f32x16 st = f32x16{0};
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) st = mfma_bf16(*reinterpret_cast<const u32x4*>(kbase + ks * 32), qf[ks], st);
+    for (int i = 0; i < KSW; ++i)
+      if (ks0 + i < KS) st = mfma_bf16(*reinterpret_cast<const u32x4*>(kbase + (ks0 + i) * 32), qf[i], st);      // wave-uniform test
+    if constexpr (SPLITK) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) sred[(wave * 16 + e) * 64 + lane] = st[e];
+      __syncthreads();
+#pragma unroll
+      for (int e = 0; e < 16; ++e)
+        st[e] = (sred[e * 64 + lane] + sred[(16 + e) * 64 + lane]) + (sred[(32 + e) * 64 + lane] + sred[(48 + e) * 64 + lane]);
+    }
     float s[16];
     float mx = -INFINITY;
 #pragma unroll
@@ -318,18 +360,19 @@ __global__ __launch_bounds__(256) void sink_group_kernel(const SinkTileArgs a, c
   l += __shfl_xor(l, 32, 64);
   if (!hvalid) return;
   if (splits > 1) {
-    float* prow = partial + ((static_cast<int64_t>(blockIdx.z) * gridDim.x + t) * a.H + head) * (a.dv + 2);
+    const int pw = partial_width(a.dv);
+    float* prow = partial + ((static_cast<int64_t>(blockIdx.z) * gridDim.x + t) * a.H + head) * pw;
 #pragma unroll
     for (int i = 0; i < DTW; ++i) {
       const int dt = wave + 4 * i;
       if (dt < DT)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const int d = dt * 32 + 8 * (e >> 2) + 4 * hb + (e & 3);
-          if (d < a.dv) prow[d] = o[i][e];
+        for (int q4 = 0; q4 < 4; ++q4) {
+          const int d = dt * 32 + 8 * q4 + 4 * hb;
+          if (d < a.dv) *reinterpret_cast<float4*>(prow + d) = float4{o[i][4 * q4], o[i][4 * q4 + 1], o[i][4 * q4 + 2], o[i][4 * q4 + 3]};
         }
     }
-    if (wave == 0 && hb == 0) { prow[a.dv] = m / LOG2E; prow[a.dv + 1] = l; }
+    if (wave == 0 && hb == 0) { prow[pw - 2] = m / LOG2E; prow[pw - 1] = l; }
     return;
   }
   float f = 1.f / l;

@@ -287,7 +287,7 @@ def sink_attention(q: torch.Tensor, k_new: torch.Tensor, v_new: torch.Tensor, ca
             keys = cache.rows
         splits = min(64, (keys + 63) // 64)
         if splits > 1:
-            partial = torch.empty((splits, t, heads, dv + 2), dtype=torch.float32, device=q.device)
+            partial = torch.empty((splits, t, heads, (dv + 3) // 4 * 4 + 4), dtype=torch.float32, device=q.device)
             a.partial, a.partial_splits = partial.data_ptr(), splits
     _lib.check_mixers(_lib.mixers().gbxm_sink_attention(ctypes.byref(a), _stream(q.device)))
     return out

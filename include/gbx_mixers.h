@@ -130,7 +130,7 @@ typedef struct {
   int32_t keep, ring;
   float scale;
   int32_t decode_only, act;
-  void* partial;                /* optional fp32 [partial_splits][T][H][dv + 2] */
+  void* partial;                /* optional fp32 [partial_splits][T][H][(dv + 3) / 4 * 4 + 4] */
   int32_t partial_splits;
 } gbxm_sink_attn_args;
 int gbxm_sink_attention(const gbxm_sink_attn_args* a, void* stream);
